@@ -46,10 +46,14 @@ def get_architecture(name: str) -> Architecture:
 
 
 def architecture_name(cfg_dict: dict) -> str:
+    """``architectures[0]``, or the single name under ``architecture``."""
     archs = cfg_dict.get("architectures")
-    if not archs or not isinstance(archs, (list, tuple)):
-        raise ConfigError("config.json: 'architectures' is missing or empty; it selects the model class")
-    return str(archs[0])
+    if archs and isinstance(archs, (list, tuple)):
+        return str(archs[0])
+    one = cfg_dict.get("architecture")
+    if isinstance(one, str) and one:
+        return one
+    raise ConfigError("config.json: 'architectures' is missing or empty; it selects the model class")
 
 
 def load_model_config(model_dir: str | os.PathLike):
@@ -60,9 +64,15 @@ def load_model_config(model_dir: str | os.PathLike):
     with open(path, "r", encoding="utf-8") as f:
         raw = json.load(f)
     arch = get_architecture(architecture_name(raw))
-    return arch, arch.config_cls.from_dict(raw)
+    config = arch.config_cls.from_dict(raw)
+    # a configuration may leave sizes to the tensors' shapes: then the checkpoint's header is read too
+    if getattr(config, "needs_shapes", lambda: False)():
+        from tensorline_amd.weights.loader import checkpoint_shapes
+        config = config.with_shapes(checkpoint_shapes(os.fspath(model_dir)))
+    return arch, config
 
 
 def _ensure_builtin() -> None:
     # Importing the module registers it; done lazily so that config/ has no import cycle.
     import tensorline_amd.models.qwen2  # noqa: F401
+    import tensorline_amd.models.samovik  # noqa: F401

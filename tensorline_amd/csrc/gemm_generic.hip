@@ -81,8 +81,11 @@ template <typename TA, typename TW, typename TO, int WM, int WN, int MB, int NB>
 __global__ __launch_bounds__(GG_THREADS) void gemm_generic_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
                                                                  const float* __restrict__ bias, TO* __restrict__ C,
                                                                  int M, int N, int K, int lda, int ldc, int a_vec,
-                                                                 int w_vec) {
+                                                                 int w_vec, long long a_bs, long long w_bs, long long c_bs) {
     constexpr int BM = WM * MB * 16, BN = WN * NB * 16;
+    A += (size_t)blockIdx.z * a_bs;          // a batch of products: one per blockIdx.z, operands a stride apart
+    W += (size_t)blockIdx.z * w_bs;
+    C += (size_t)blockIdx.z * c_bs;
     constexpr int A_PIECES = BM * 4, W_PIECES = BN * 4;                 // 16-byte (four k) pieces per step
     constexpr int A_PER = (A_PIECES + GG_THREADS - 1) / GG_THREADS, W_PER = (W_PIECES + GG_THREADS - 1) / GG_THREADS;
     __shared__ float As[2][BM * GG_LD];
@@ -207,8 +210,12 @@ static inline int gf_waves(int nseg, int tiles) {
 template <typename TA, typename TW, typename TO, bool SHUF>
 __global__ __launch_bounds__(GF_WAVES * 64) void gemm_fewrows_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
                                                            const float* __restrict__ bias, TO* __restrict__ C, int M,
-                                                           int N, int K, int lda, int ldc, int a_vec, int w_vec) {
-    extern __shared__ float gf_part[];                       // [segment][register v][lane]
+                                                           int N, int K, int lda, int ldc, int a_vec, int w_vec,
+                                                           long long a_bs, long long w_bs, long long c_bs) {
+    extern __shared__ float gf_part[];
+    A += (size_t)blockIdx.y * a_bs;          // a batch of products: one per blockIdx.y
+    W += (size_t)blockIdx.y * w_bs;
+    C += (size_t)blockIdx.y * c_bs;                       // [segment][register v][lane]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
     const int n0 = blockIdx.x * 16;
@@ -287,25 +294,25 @@ __global__ __launch_bounds__(GF_WAVES * 64) void gemm_fewrows_kernel(const TA* _
 
 template <typename TA, typename TW, typename TO>
 static int gg_launch(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, int lda, int ldc,
-                     hipStream_t stream) {
+                     hipStream_t stream, int batch = 1, long long a_bs = 0, long long w_bs = 0, long long c_bs = 0) {
     // whole 16-byte (8-byte for bfloat16) pieces can be read where rows start aligned
-    const int a_vec = ((uintptr_t)A % (4 * sizeof(TA)) == 0 && lda % 4 == 0) ? 1 : 0;
-    const int w_vec = ((uintptr_t)W % (4 * sizeof(TW)) == 0 && K % 4 == 0) ? 1 : 0;
+    const int a_vec = ((uintptr_t)A % (4 * sizeof(TA)) == 0 && lda % 4 == 0 && a_bs % 4 == 0) ? 1 : 0;
+    const int w_vec = ((uintptr_t)W % (4 * sizeof(TW)) == 0 && K % 4 == 0 && w_bs % 4 == 0) ? 1 : 0;
 #define GG_GO(WM, WN, MB, NB)                                                                                    \
     do {                                                                                                         \
         constexpr int BM = WM * MB * 16, BN = WN * NB * 16;                                                      \
         const long long gy = tl_ceil_div(M, BM);                                                                 \
         if (gy > 65535) return tl_fail("tl_gemm_generic: %d rows are too many for one launch", M);               \
-        dim3 grid(tl_ceil_div(N, BN), (unsigned)gy), block(GG_THREADS);                                          \
+        dim3 grid(tl_ceil_div(N, BN), (unsigned)gy, batch), block(GG_THREADS);                                   \
         hipLaunchKernelGGL((gemm_generic_kernel<TA, TW, TO, WM, WN, MB, NB>), grid, block, 0, stream,            \
-                           (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec);           \
+                           (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec, a_bs, w_bs, c_bs); \
     } while (0)
     const int nseg = tl_ceil_div(K, GF_SEG);
     if (M <= 16 && nseg <= GF_MAX_SEGMENTS) {
         const int waves = gf_waves(nseg, tl_ceil_div(N, 16));
         const size_t lds = (size_t)nseg * 4 * 64 * sizeof(float);
-        hipLaunchKernelGGL((gemm_fewrows_kernel<TA, TW, TO, false>), dim3(tl_ceil_div(N, 16)), dim3(64 * waves), lds, stream,
-                           (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec);
+        hipLaunchKernelGGL((gemm_fewrows_kernel<TA, TW, TO, false>), dim3(tl_ceil_div(N, 16), batch), dim3(64 * waves), lds, stream,
+                           (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec, a_bs, w_bs, c_bs);
     } else if (M <= 32)
         GG_GO(1, 4, 2, 1);        // 32 x 64
     else if (M <= 64)
@@ -334,7 +341,7 @@ extern "C" int tl_gemm_fewrows_shuffled(const float* A, const float* Ws, const f
     const int waves = gf_waves(nseg, tl_ceil_div(N, 16));
     const size_t lds = (size_t)nseg * 4 * 64 * sizeof(float);
     hipLaunchKernelGGL((gemm_fewrows_kernel<float, float, float, true>), dim3(tl_ceil_div(N, 16)), dim3(64 * waves), lds, stream,
-                       A, Ws, bias, C, M, N, K, lda, ldc, a_vec, 1);
+                       A, Ws, bias, C, M, N, K, lda, ldc, a_vec, 1, 0LL, 0LL, 0LL);
     TL_CHECK_LAUNCH("tl_gemm_fewrows_shuffled");
     return 0;
 }
@@ -358,5 +365,27 @@ extern "C" int tl_gemm_generic(const void* A, int a_dtype, const void* W, int w_
         return tl_fail("tl_gemm_generic: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
     if (rc) return rc;
     TL_CHECK_LAUNCH("tl_gemm_generic");
+    return 0;
+}
+
+// `batch` products of the same shape in one launch: product b reads A + b * a_bs (row stride lda),
+// W + b * w_bs ([N, K] contiguous) and writes C + b * c_bs (row stride ldc); strides in elements.
+// Each is summed as tl_gemm_generic sums it.  (A head's share of a projection that is applied per
+// head: the operands are column blocks of wider matrices, a stride of one head apart.)
+extern "C" int tl_gemm_generic_batched(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M,
+                                       int N, int K, int lda, int ldc, int batch, long long a_bs, long long w_bs,
+                                       long long c_bs, hipStream_t stream) {
+    TL_CHECK_ARG(M >= 0 && N > 0 && K > 0 && batch > 0 && batch <= 65535, "tl_gemm_generic_batched: bad sizes M=%d N=%d K=%d batch=%d", M, N, K, batch);
+    TL_CHECK_ARG(lda >= K && ldc >= N, "tl_gemm_generic_batched: row strides lda=%d ldc=%d too small for K=%d N=%d", lda, ldc, K, N);
+    if (M == 0) return 0;
+    int rc;
+    if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32)
+        rc = gg_launch<float, float, float>(A, W, nullptr, C, M, N, K, lda, ldc, stream, batch, a_bs, w_bs, c_bs);
+    else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_BF16)
+        rc = gg_launch<bf16_t, bf16_t, bf16_t>(A, W, nullptr, C, M, N, K, lda, ldc, stream, batch, a_bs, w_bs, c_bs);
+    else
+        return tl_fail("tl_gemm_generic_batched: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
+    if (rc) return rc;
+    TL_CHECK_LAUNCH("tl_gemm_generic_batched");
     return 0;
 }

@@ -1,0 +1,323 @@
+// Routed experts: choice of experts per token, the tokens of each expert gathered into row tiles,
+// the experts' products as one grouped launch each, and the weighted sum per token.
+//
+//   tl_moe_route    per token: the `top` largest router logits (lowest index wins a tie) and the
+//                   softmax over those alone                      -> expert ids, weights [T, top]
+//   tl_moe_sort     the (token, choice) pairs ordered by expert and cut into row tiles of BM rows that
+//                   hold one expert's pairs only                 -> order, tiles
+//   tl_moe_gemm     a product per tile with its expert's matrix: gate/up with the clamped gated
+//                   activation in the epilogue, or down, which scatters rows back to their pairs
+//   tl_moe_combine  out[t] = sum over the token's choices, in the order of its choices, of weight *
+//                   row (+ a shared expert's output)
+//
+// A pair's row is computed alone (a row of a tile does not see the other rows) and summed over k in
+// one fixed order, and a token's choices are added in one fixed order, so neither the batch nor the
+// place a pair gets inside its expert's tiles changes a bit of a result.  The products run on the
+// float matrix instruction (v_mfma_f32_16x16x4_f32), bfloat16 operands widened on the way into
+// LDS, as the any-shape product does.
+#include "common.h"
+
+#include <math.h>
+
+#define MOE_MAX_EXPERTS 1024
+#define MOE_MAX_TOP 32
+
+// ---- routing ------------------------------------------------------------------------------------------
+__global__ void moe_route_kernel(const float* __restrict__ logits, int ldl, int32_t* __restrict__ ids,
+                                 float* __restrict__ weights, int T, int E, int top) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= T) return;
+    const float* z = logits + (size_t)t * ldl;
+    int chosen[MOE_MAX_TOP];
+    float val[MOE_MAX_TOP];
+    for (int c = 0; c < top; ++c) {
+        int best = -1;
+        float bv = 0.f;
+        for (int e = 0; e < E; ++e) {
+            bool taken = false;
+            for (int p = 0; p < c; ++p) taken |= chosen[p] == e;
+            if (taken) continue;
+            const float v = z[e];
+            if (best < 0 || v > bv || (v != v && bv == bv)) {      // a NaN logit is chosen, so that it shows
+                best = e;
+                bv = v;
+            }
+        }
+        chosen[c] = best;
+        val[c] = bv;
+    }
+    float sum = 0.f;
+    const float largest = val[0];
+    for (int c = 0; c < top; ++c) {
+        val[c] = expf(val[c] - largest);
+        sum += val[c];
+    }
+    for (int c = 0; c < top; ++c) {
+        ids[(size_t)t * top + c] = chosen[c];
+        weights[(size_t)t * top + c] = val[c] / sum;
+    }
+}
+
+extern "C" int tl_moe_route(const float* logits, int ldl, int32_t* ids, float* weights, int T, int E, int top,
+                            hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && E > 0 && top > 0 && top <= E && top <= MOE_MAX_TOP && ldl >= E, "tl_moe_route: bad sizes E=%d top=%d", E, top);
+    if (T == 0) return 0;
+    hipLaunchKernelGGL(moe_route_kernel, dim3(tl_ceil_div(T, 64)), dim3(64), 0, stream, logits, ldl, ids, weights, T, E, top);
+    TL_CHECK_LAUNCH("tl_moe_route");
+    return 0;
+}
+
+// ---- pairs ordered by expert ----------------------------------------------------------------------------
+// P = T * top pairs.  order[P]: the pair at each place; places of an expert are consecutive.  A tile
+// is (expert, first place, rows); tiles[0] = number of tiles, then three ints per tile.  One
+// work-group; counts and cursors in LDS.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ order,
+                                                         int32_t* __restrict__ tiles, int P, int E, int BM) {
+    __shared__ int count[MOE_MAX_EXPERTS], first[MOE_MAX_EXPERTS], tile0[MOE_MAX_EXPERTS + 1];
+    for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < P; p += blockDim.x) {
+        const int e = ids[p];
+        if (e >= 0 && e < E) atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, nt = 0;
+        for (int e = 0; e < E; ++e) {
+            first[e] = at;
+            tile0[e] = nt;
+            at += count[e];
+            nt += (count[e] + BM - 1) / BM;
+        }
+        tile0[E] = nt;
+        tiles[0] = nt;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        const int n = count[e];
+        for (int i = 0, tl = tile0[e]; i < n; i += BM, ++tl) {
+            tiles[1 + 3 * tl] = e;
+            tiles[2 + 3 * tl] = first[e] + i;
+            tiles[3 + 3 * tl] = min(BM, n - i);
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;      // now the cursor within the expert
+    __syncthreads();
+    for (int p = threadIdx.x; p < P; p += blockDim.x) {
+        const int e = ids[p];
+        if (e >= 0 && e < E) order[first[e] + atomicAdd(&count[e], 1)] = p;
+    }
+}
+
+extern "C" int tl_moe_sort(const int32_t* ids, int32_t* order, int32_t* tiles, int P, int E, int BM, hipStream_t stream) {
+    TL_CHECK_ARG(P >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && (BM == 16 || BM == 64), "tl_moe_sort: bad sizes P=%d E=%d BM=%d", P, E, BM);
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(P >= 1024 ? 1024 : 256), 0, stream, ids, order, tiles, P, E, BM);
+    TL_CHECK_LAUNCH("tl_moe_sort");
+    return 0;
+}
+
+// ---- the grouped product ----------------------------------------------------------------------------------
+#define MG_THREADS 256
+#define MG_KS 16
+#define MG_LD (MG_KS + 4)
+typedef float mg_f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> __device__ __forceinline__ float4 mg_load4(const T* __restrict__ base, bool ok, int k, int K, bool vec);
+template <> __device__ __forceinline__ float4 mg_load4<float>(const float* __restrict__ base, bool ok, int k, int K, bool vec) {
+    if (!ok || k >= K) return make_float4(0.f, 0.f, 0.f, 0.f);
+    if (vec && k + 3 < K) return *reinterpret_cast<const float4*>(base + k);
+    float4 r;
+    r.x = base[k];
+    r.y = (k + 1 < K) ? base[k + 1] : 0.f;
+    r.z = (k + 2 < K) ? base[k + 2] : 0.f;
+    r.w = (k + 3 < K) ? base[k + 3] : 0.f;
+    return r;
+}
+template <> __device__ __forceinline__ float4 mg_load4<bf16_t>(const bf16_t* __restrict__ base, bool ok, int k, int K, bool vec) {
+    if (!ok || k >= K) return make_float4(0.f, 0.f, 0.f, 0.f);
+    if (vec && k + 3 < K) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(base + k);
+        return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                           __uint_as_float(raw.y & 0xffff0000u));
+    }
+    float4 r;
+    r.x = tl_to_float(base[k]);
+    r.y = (k + 1 < K) ? tl_to_float(base[k + 1]) : 0.f;
+    r.z = (k + 2 < K) ? tl_to_float(base[k + 2]) : 0.f;
+    r.w = (k + 3 < K) ? tl_to_float(base[k + 3]) : 0.f;
+    return r;
+}
+
+// GLU: W [E, 2 N, K] (gate rows, then up rows), A rows are the tokens of the tile's pairs
+// (order[place] / top), C [P, N] by place, C = act(gate, up).  Otherwise: W [E, N, K], A [P, K] by
+// place, C [P, N] by pair (order[place]).  Four waves side by side, each MB x NB blocks of 16 x 16
+// (GLU: NB gate blocks and NB up blocks).
+template <typename TA, typename TW, typename TO, int MB, int NB, bool GLU>
+__global__ __launch_bounds__(MG_THREADS) void moe_gemm_kernel(const TA* __restrict__ A, int lda, const TW* __restrict__ W,
+                                                             TO* __restrict__ C, int ldc, const int32_t* __restrict__ order,
+                                                             const int32_t* __restrict__ tiles, int top, int N, int K,
+                                                             int a_vec, int w_vec, float limit, float alpha) {
+    constexpr int BM = MB * 16, BN = 4 * NB * 16, WR = GLU ? 2 * BN : BN, NW = GLU ? 2 * NB : NB;
+    constexpr int A_PIECES = BM * 4, W_PIECES = WR * 4;
+    constexpr int A_PER = (A_PIECES + MG_THREADS - 1) / MG_THREADS, W_PER = (W_PIECES + MG_THREADS - 1) / MG_THREADS;
+    __shared__ float As[2][BM * MG_LD];
+    __shared__ float Ws[2][WR * MG_LD];
+    __shared__ int arow[BM];
+    if ((int)blockIdx.y >= tiles[0]) return;
+    const int e = tiles[1 + 3 * blockIdx.y], place0 = tiles[2 + 3 * blockIdx.y], rows = tiles[3 + 3 * blockIdx.y];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+    const int n0 = blockIdx.x * BN;
+    for (int r = tid; r < BM; r += MG_THREADS) arow[r] = r < rows ? (GLU ? order[place0 + r] / top : place0 + r) : -1;
+    __syncthreads();
+    const TW* We = W + (size_t)e * (GLU ? 2 : 1) * N * K;
+
+    mg_f32x4 acc[MB][NW];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NW; ++j) acc[i][j] = (mg_f32x4){0.f, 0.f, 0.f, 0.f};
+
+    float4 areg[A_PER], wreg[W_PER];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int it = 0; it < A_PER; ++it) {
+            const int p = tid + it * MG_THREADS;
+            const int r = p >> 2, c4 = p & 3;
+            const int src = p < A_PIECES ? arow[r] : -1;
+            areg[it] = mg_load4<TA>(A + (size_t)(src < 0 ? 0 : src) * lda, src >= 0, k0 + 4 * c4, K, a_vec != 0);
+        }
+#pragma unroll
+        for (int it = 0; it < W_PER; ++it) {
+            const int p = tid + it * MG_THREADS;
+            const int r = p >> 2, c4 = p & 3;
+            // LDS row r: gate (or plain) row n0 + r for r < BN, up row N + n0 + r - BN beyond
+            const int col = (GLU && r >= BN) ? n0 + r - BN : n0 + r;
+            const size_t wrow = (GLU && r >= BN) ? (size_t)N + col : (size_t)col;
+            wreg[it] = mg_load4<TW>(We + wrow * K, p < W_PIECES && col < N, k0 + 4 * c4, K, w_vec != 0);
+        }
+    };
+    auto to_lds = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < A_PER; ++it) {
+            const int p = tid + it * MG_THREADS;
+            if (p < A_PIECES) *reinterpret_cast<float4*>(&As[buf][(p >> 2) * MG_LD + 4 * (p & 3)]) = areg[it];
+        }
+#pragma unroll
+        for (int it = 0; it < W_PER; ++it) {
+            const int p = tid + it * MG_THREADS;
+            if (p < W_PIECES) *reinterpret_cast<float4*>(&Ws[buf][(p >> 2) * MG_LD + 4 * (p & 3)]) = wreg[it];
+        }
+    };
+
+    fetch(0);
+    to_lds(0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += MG_KS) {
+        const bool more = k0 + MG_KS < K;
+        if (more) fetch(k0 + MG_KS);
+        float4 af[MB], wf[NW];
+#pragma unroll
+        for (int i = 0; i < MB; ++i) af[i] = *reinterpret_cast<const float4*>(&As[buf][(i * 16 + li) * MG_LD + 4 * lg]);
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+            const int r = (j < NB ? 0 : BN) + (wave * NB + (j < NB ? j : j - NB)) * 16 + li;
+            wf[j] = *reinterpret_cast<const float4*>(&Ws[buf][r * MG_LD + 4 * lg]);
+        }
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+            for (int j = 0; j < NW; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i].x, wf[j].x, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i].y, wf[j].y, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i].z, wf[j].z, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i].w, wf[j].w, acc[i][j], 0, 0, 0);
+            }
+        if (more) {
+            to_lds(buf ^ 1);
+            __syncthreads();
+            buf ^= 1;
+        }
+    }
+
+    // this lane holds rows 4 lg + v and column li of each block
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int n = n0 + (wave * NB + j) * 16 + li;
+        if (n >= N) continue;
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int r = i * 16 + 4 * lg + v;
+                if (r >= rows) continue;
+                if (GLU) {
+                    const float g = fminf(acc[i][j][v], limit);
+                    const float u = fminf(fmaxf(acc[i][NB + j][v], -limit), limit);
+                    C[(size_t)(place0 + r) * ldc + n] = tl_from_float<TO>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
+                } else {
+                    C[(size_t)order[place0 + r] * ldc + n] = tl_from_float<TO>(acc[i][j][v]);
+                }
+            }
+    }
+}
+
+// glu 1: A [T, K] tokens (row stride lda), W [E, 2N, K], C [P, N] by place, of type c_dtype.
+// glu 0: A [P, K] by place, W [E, N, K], C float [P, N] by pair.  max_tiles bounds the tiles that
+// tl_moe_sort can have made: P / BM + E.
+extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, int w_dtype, void* C, int c_dtype, int ldc,
+                           const int32_t* order, const int32_t* tiles, int max_tiles, int BM, int top, int N, int K, int glu,
+                           float limit, float alpha, hipStream_t stream) {
+    TL_CHECK_ARG(N > 0 && K > 0 && lda >= K && ldc >= N && top > 0 && (BM == 16 || BM == 64), "tl_moe_gemm: bad sizes N=%d K=%d BM=%d", N, K, BM);
+    TL_CHECK_ARG(max_tiles >= 0 && max_tiles <= 65535, "tl_moe_gemm: %d row tiles are too many for one launch", max_tiles);
+    if (max_tiles == 0) return 0;
+    const size_t a_el = a_dtype == TL_F32 ? 4 : 2, w_el = w_dtype == TL_F32 ? 4 : 2;
+    const int a_vec = ((uintptr_t)A % (4 * a_el) == 0 && lda % 4 == 0) ? 1 : 0;
+    const int w_vec = ((uintptr_t)W % (4 * w_el) == 0 && K % 4 == 0) ? 1 : 0;
+#define GO(TA, TW, TO, MB, NB, GLU)                                                                                       \
+    hipLaunchKernelGGL((moe_gemm_kernel<TA, TW, TO, MB, NB, GLU>), dim3(tl_ceil_div(N, 4 * NB * 16), max_tiles),          \
+                       dim3(MG_THREADS), 0, stream, (const TA*)A, lda, (const TW*)W, (TO*)C, ldc, order, tiles, top, N, K, \
+                       a_vec, w_vec, limit, alpha)
+#define GO_BM(TA, TW, TO, GLU)                 \
+    do {                                       \
+        if (BM == 16) GO(TA, TW, TO, 1, 1, GLU); \
+        else GO(TA, TW, TO, 4, 1, GLU);          \
+    } while (0)
+    if (glu) {
+        if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32) GO_BM(float, float, float, true);
+        else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_BF16) GO_BM(bf16_t, bf16_t, bf16_t, true);
+        else return tl_fail("tl_moe_gemm: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
+    } else {
+        if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32) GO_BM(float, float, float, false);
+        else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_F32) GO_BM(bf16_t, bf16_t, float, false);
+        else return tl_fail("tl_moe_gemm: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
+    }
+#undef GO_BM
+#undef GO
+    TL_CHECK_LAUNCH("tl_moe_gemm");
+    return 0;
+}
+
+// ---- the weighted sum per token ---------------------------------------------------------------------------------
+__global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ weights,
+                                   const float* __restrict__ shared, float* __restrict__ out, int T, int N, int top) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)T * N) return;
+    const size_t t = i / N, c = i - t * N;
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) sum += weights[t * top + k] * y[(t * top + k) * N + c];
+    if (shared) sum += shared[i];
+    out[i] = sum;
+}
+
+extern "C" int tl_moe_combine(const float* y, const float* weights, const float* shared, float* out, int T, int N, int top,
+                              hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && N > 0 && top > 0, "tl_moe_combine: bad sizes");
+    if (T == 0) return 0;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)(((size_t)T * N + 255) / 256)), dim3(256), 0, stream, y, weights,
+                       shared, out, T, N, top);
+    TL_CHECK_LAUNCH("tl_moe_combine");
+    return 0;
+}

@@ -1,0 +1,362 @@
+// Row-wise and element-wise kernels of the mixers and feed-forwards that are not plain attention
+// and SwiGLU: the Dynamic Tanh norm, the clamped gated activation of routed experts, gated
+// normalisation over groups of columns, the token shift of time-mixing layers, the per-layer token
+// input, and what a latent-attention step does between its projections and the attention kernel.
+//
+// As everywhere: the residual stream is float; activations between kernels are float or bfloat16
+// (template argument); all arithmetic is float.
+#include "common.h"
+
+#include <math.h>
+
+template <typename T> __device__ __forceinline__ float pw_read(const void* p, size_t i) {
+    return tl_to_float(reinterpret_cast<const T*>(p)[i]);
+}
+template <typename T> __device__ __forceinline__ void pw_write(void* p, size_t i, float v) {
+    reinterpret_cast<T*>(p)[i] = tl_from_float<T>(v);
+}
+
+__device__ __forceinline__ float pw_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float pw_silu(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float pw_gelu_tanh(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// ---- residual add + Dynamic Tanh ---------------------------------------------------------------
+// Without `rows`: x[r] += residual[r] (float, written back); out[r] = tanh(alpha x[r]) * w + b.
+// With `rows`: the same for x[rows[r]] + residual[rows[r]], x untouched.  No statistic of the row
+// is taken, so one thread does one element.
+template <typename R, typename O>
+__global__ void add_dyt_kernel(float* __restrict__ x, const R* __restrict__ res, const float* __restrict__ w,
+                               const float* __restrict__ b, const float* __restrict__ alpha, O* __restrict__ out,
+                               const int32_t* __restrict__ rows, int H) {
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    const float a = alpha[0];
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = x[src * H + c];
+        if (res) {
+            v += tl_to_float(res[src * H + c]);
+            if (!rows) x[src * H + c] = v;
+        }
+        out[(size_t)r * H + c] = tl_from_float<O>(tanhf(a * v) * w[c] + b[c]);
+    }
+}
+
+extern "C" int tl_add_dyt(float* x, const void* res, int res_dtype, const float* w, const float* b, const float* alpha,
+                          void* out, int out_dtype, const int32_t* rows, int n, int H, hipStream_t stream) {
+    TL_CHECK_ARG(n >= 0 && H > 0, "tl_add_dyt: bad sizes n=%d H=%d", n, H);
+    if (n == 0) return 0;
+    dim3 grid(n), block(H >= 1024 ? 256 : 128);
+#define GO(R, O) hipLaunchKernelGGL((add_dyt_kernel<R, O>), grid, block, 0, stream, x, (const R*)res, w, b, alpha, (O*)out, rows, H)
+    if (res_dtype == TL_F32 && out_dtype == TL_F32) GO(float, float);
+    else if (res_dtype == TL_F32 && out_dtype == TL_BF16) GO(float, bf16_t);
+    else if (res_dtype == TL_BF16 && out_dtype == TL_F32) GO(bf16_t, float);
+    else if (res_dtype == TL_BF16 && out_dtype == TL_BF16) GO(bf16_t, bf16_t);
+    else return tl_fail("tl_add_dyt: unknown dtypes %d %d", res_dtype, out_dtype);
+#undef GO
+    TL_CHECK_LAUNCH("tl_add_dyt");
+    return 0;
+}
+
+// ---- x += residual, and x again in the activation type -------------------------------------------
+template <typename O>
+__global__ void add_cast_kernel(float* __restrict__ x, const float* __restrict__ res, O* __restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = x[i];
+    if (res) {
+        v += res[i];
+        x[i] = v;
+    }
+    out[i] = tl_from_float<O>(v);
+}
+
+extern "C" int tl_add_cast(float* x, const float* res, void* out, int out_dtype, long long n, hipStream_t stream) {
+    TL_CHECK_ARG(n >= 0, "tl_add_cast: bad size");
+    if (n == 0) return 0;
+    dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (out_dtype == TL_F32) hipLaunchKernelGGL(add_cast_kernel<float>, grid, block, 0, stream, x, res, (float*)out, (size_t)n);
+    else if (out_dtype == TL_BF16) hipLaunchKernelGGL(add_cast_kernel<bf16_t>, grid, block, 0, stream, x, res, (bf16_t*)out, (size_t)n);
+    else return tl_fail("tl_add_cast: unknown dtype %d", out_dtype);
+    TL_CHECK_LAUNCH("tl_add_cast");
+    return 0;
+}
+
+// ---- element-wise functions ------------------------------------------------------------------------
+// kind 0: tanh.  float in, float or bfloat16 out.
+template <typename O>
+__global__ void unary_kernel(const float* __restrict__ in, O* __restrict__ out, size_t n, int kind) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    out[i] = tl_from_float<O>(tanhf(in[i]));
+}
+
+extern "C" int tl_unary(const float* in, void* out, int out_dtype, long long n, int kind, hipStream_t stream) {
+    TL_CHECK_ARG(n >= 0 && kind == 0, "tl_unary: bad arguments");
+    if (n == 0) return 0;
+    dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (out_dtype == TL_F32) hipLaunchKernelGGL(unary_kernel<float>, grid, block, 0, stream, in, (float*)out, (size_t)n, kind);
+    else if (out_dtype == TL_BF16) hipLaunchKernelGGL(unary_kernel<bf16_t>, grid, block, 0, stream, in, (bf16_t*)out, (size_t)n, kind);
+    else return tl_fail("tl_unary: unknown dtype %d", out_dtype);
+    TL_CHECK_LAUNCH("tl_unary");
+    return 0;
+}
+
+// ---- clamped gated activation ------------------------------------------------------------------------
+// gu [T, 2F] (gate columns first): g = min(gate, limit), u = clamp(up, -limit, limit),
+// out = g * sigmoid(alpha g) * (u + 1).
+__device__ __forceinline__ float pw_clamp_glu(float g, float u, float limit, float alpha) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * pw_sigmoid(alpha * g) * (u + 1.0f);
+}
+
+template <typename I, typename O>
+__global__ void clamp_glu_kernel(const I* __restrict__ gu, O* __restrict__ out, int T, int F, float limit, float alpha) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)T * F) return;
+    const size_t t = i / F, c = i - t * F;
+    out[i] = tl_from_float<O>(pw_clamp_glu(tl_to_float(gu[t * 2 * F + c]), tl_to_float(gu[t * 2 * F + F + c]), limit, alpha));
+}
+
+extern "C" int tl_clamp_glu(const void* gu, int in_dtype, void* out, int out_dtype, int T, int F, float limit, float alpha,
+                            hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && F > 0, "tl_clamp_glu: bad sizes");
+    if (T == 0) return 0;
+    dim3 grid((unsigned)(((size_t)T * F + 255) / 256)), block(256);
+#define GO(I, O) hipLaunchKernelGGL((clamp_glu_kernel<I, O>), grid, block, 0, stream, (const I*)gu, (O*)out, T, F, limit, alpha)
+    if (in_dtype == TL_F32 && out_dtype == TL_F32) GO(float, float);
+    else if (in_dtype == TL_F32 && out_dtype == TL_BF16) GO(float, bf16_t);
+    else if (in_dtype == TL_BF16 && out_dtype == TL_BF16) GO(bf16_t, bf16_t);
+    else return tl_fail("tl_clamp_glu: unsupported dtypes %d %d", in_dtype, out_dtype);
+#undef GO
+    TL_CHECK_LAUNCH("tl_clamp_glu");
+    return 0;
+}
+
+// ---- gated normalisation over groups of columns ----------------------------------------------------
+// o float [T, N] in groups of `group` columns (a head, or the whole row): every group is divided by
+// its root mean square (eps inside the root), times weight[c], times the gate: sigmoid(gate) for
+// gate_act 0, silu(gate) for 1.  gate float [T, ldg].  One wave per group.
+template <typename O>
+__global__ void gated_group_norm_kernel(const float* __restrict__ o, int ldo, const float* __restrict__ weight,
+                                        const float* __restrict__ gate, int ldg, O* __restrict__ out, int N, int group,
+                                        float eps, int gate_act) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int groups = N / group;
+    for (int g = wave; g < groups; g += nwaves) {
+        const float* row = o + (size_t)t * ldo + g * group;
+        float ss = 0.f;
+        for (int c = lane; c < group; c += 64) ss += row[c] * row[c];
+        ss = tl_wave_sum(ss);
+        const float rstd = 1.0f / sqrtf(ss / (float)group + eps);
+        for (int c = lane; c < group; c += 64) {
+            const int n = g * group + c;
+            const float z = gate[(size_t)t * ldg + n];
+            const float gv = gate_act == 0 ? pw_sigmoid(z) : pw_silu(z);
+            out[(size_t)t * N + n] = tl_from_float<O>(row[c] * rstd * weight[n] * gv);
+        }
+    }
+}
+
+extern "C" int tl_gated_group_norm(const float* o, int ldo, const float* weight, const float* gate, int ldg, void* out,
+                                   int out_dtype, int T, int N, int group, float eps, int gate_act, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && N > 0 && group > 0 && N % group == 0 && ldo >= N && ldg >= N, "tl_gated_group_norm: bad sizes");
+    if (T == 0) return 0;
+    const int groups = N / group;
+    dim3 grid(T), block(64 * (groups < 4 ? groups : 4));
+    if (out_dtype == TL_F32)
+        hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, 0, stream, o, ldo, weight, gate, ldg, (float*)out, N, group, eps, gate_act);
+    else if (out_dtype == TL_BF16)
+        hipLaunchKernelGGL(gated_group_norm_kernel<bf16_t>, grid, block, 0, stream, o, ldo, weight, gate, ldg, (bf16_t*)out, N, group, eps, gate_act);
+    else return tl_fail("tl_gated_group_norm: unknown dtype %d", out_dtype);
+    TL_CHECK_LAUNCH("tl_gated_group_norm");
+    return 0;
+}
+
+// ---- token shift -------------------------------------------------------------------------------------
+// h [T, W]: out[s][t] = h[t] + (before[t] - h[t]) * mu[s] for `ways` mixing vectors mu [ways, W], where
+// before[t] is the row above in the same sequence, and for a sequence's first row of this step the row
+// kept in its state slot (zeros for a new request).  prev: float, the slot's row at prev + slot * stride.
+template <typename T>
+__global__ void token_shift_kernel(const T* __restrict__ h, const int32_t* __restrict__ seq_of_token,
+                                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
+                                   const float* __restrict__ prev, long long stride, const float* __restrict__ mu,
+                                   T* __restrict__ out, int Tn, int W, int ways) {
+    const int t = blockIdx.x;
+    const int s = seq_of_token[t];
+    const bool first = q_start[s] == t;
+    const float* pr = prev + (size_t)state_slots[s] * stride;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float cur = tl_to_float(h[(size_t)t * W + c]);
+        const float bef = first ? pr[c] : tl_to_float(h[(size_t)(t - 1) * W + c]);
+        const float d = bef - cur;
+        for (int m = 0; m < ways; ++m) out[((size_t)m * Tn + t) * W + c] = tl_from_float<T>(cur + d * mu[(size_t)m * W + c]);
+    }
+}
+
+// The last row each sequence brought becomes the row its slot keeps.  Runs after the kernel above.
+template <typename T>
+__global__ void token_shift_keep_kernel(const T* __restrict__ h, const int32_t* __restrict__ q_start,
+                                        const int32_t* __restrict__ state_slots, float* __restrict__ prev, long long stride, int W) {
+    const int s = blockIdx.x;
+    const int last = q_start[s + 1] - 1;
+    if (last < q_start[s]) return;
+    float* pr = prev + (size_t)state_slots[s] * stride;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) pr[c] = tl_to_float(h[(size_t)last * W + c]);
+}
+
+extern "C" int tl_token_shift(const void* h, int dtype, const int32_t* seq_of_token, const int32_t* q_start,
+                              const int32_t* state_slots, float* prev, long long stride, const float* mu, void* out, int T,
+                              int S, int W, int ways, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && S > 0 && W > 0 && ways > 0 && stride >= W, "tl_token_shift: bad sizes");
+    if (T == 0) return 0;
+    dim3 block(W >= 1024 ? 256 : 128);
+    if (dtype == TL_F32) {
+        hipLaunchKernelGGL(token_shift_kernel<float>, dim3(T), block, 0, stream, (const float*)h, seq_of_token, q_start, state_slots, prev, stride, mu, (float*)out, T, W, ways);
+        hipLaunchKernelGGL(token_shift_keep_kernel<float>, dim3(S), block, 0, stream, (const float*)h, q_start, state_slots, prev, stride, W);
+    } else if (dtype == TL_BF16) {
+        hipLaunchKernelGGL(token_shift_kernel<bf16_t>, dim3(T), block, 0, stream, (const bf16_t*)h, seq_of_token, q_start, state_slots, prev, stride, mu, (bf16_t*)out, T, W, ways);
+        hipLaunchKernelGGL(token_shift_keep_kernel<bf16_t>, dim3(S), block, 0, stream, (const bf16_t*)h, q_start, state_slots, prev, stride, W);
+    } else return tl_fail("tl_token_shift: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_token_shift");
+    return 0;
+}
+
+// ---- per-layer token input: gate ---------------------------------------------------------------------
+// out[t, c] = gelu_tanh(z[t, c]) * table[ids[t], col0 + c]; z float [T, D], table [V, ld].
+template <typename T>
+__global__ void gelu_token_gate_kernel(const float* __restrict__ z, const T* __restrict__ table, const int32_t* __restrict__ ids,
+                                       T* __restrict__ out, int D, int ld, int col0, int V) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    for (int c = threadIdx.x; c < D; c += blockDim.x) {
+        const float e = (id >= 0 && id < V) ? tl_to_float(table[(size_t)id * ld + col0 + c]) : NAN;
+        out[(size_t)t * D + c] = tl_from_float<T>(pw_gelu_tanh(z[(size_t)t * D + c]) * e);
+    }
+}
+
+extern "C" int tl_gelu_token_gate(const float* z, const void* table, int dtype, const int32_t* ids, void* out, int T, int D,
+                                  int ld, int col0, int V, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && D > 0 && col0 >= 0 && col0 + D <= ld && V > 0, "tl_gelu_token_gate: bad sizes");
+    if (T == 0) return 0;
+    dim3 grid(T), block(D >= 256 ? 256 : 64);
+    if (dtype == TL_F32) hipLaunchKernelGGL(gelu_token_gate_kernel<float>, grid, block, 0, stream, z, (const float*)table, ids, (float*)out, D, ld, col0, V);
+    else if (dtype == TL_BF16) hipLaunchKernelGGL(gelu_token_gate_kernel<bf16_t>, grid, block, 0, stream, z, (const bf16_t*)table, ids, (bf16_t*)out, D, ld, col0, V);
+    else return tl_fail("tl_gelu_token_gate: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_gelu_token_gate");
+    return 0;
+}
+
+// ---- latent attention: between the projections and the attention kernel ---------------------------------
+// proj float [T, ldp] holds per token: H query heads of (d plain + r rotated) columns, then the
+// compressed row of `rank` columns and r columns of the one rotated key part all heads share.
+// Per token (one work-group):
+//   * the compressed row is divided by its root mean square (eps inside the root) and scaled by
+//     norm_w: the latent c;
+//   * query and key rotated parts are turned: pair (i, i + r/2) by the angle pos * freq[i], cosine and
+//     sine both times `mag`;
+//   * plain query parts go to q_plain [T, H*d];
+//   * rotated query parts go to q_lat [T, H*D] at columns [rank, rank + r) of each head, zeros up to D
+//     (the first `rank` columns are written by the product with the key expansion);
+//   * the row [c | rotated key part | zeros] of D columns goes into the cache at `slot`, once token-major
+//     ([pages, page, 1, D]) and once with a page's tokens innermost ([pages, 1, D, page]).
+template <typename T>
+__global__ void latent_prepare_kernel(const float* __restrict__ proj, int ldp, const int32_t* __restrict__ pos,
+                                      const float* __restrict__ freq, float mag, const float* __restrict__ norm_w, float eps,
+                                      const int32_t* __restrict__ slots, T* __restrict__ q_plain, T* __restrict__ q_lat,
+                                      T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int d, int r, int rank, int D,
+                                      int page) {
+    __shared__ float red[16];
+    const int t = blockIdx.x;
+    const float* row = proj + (size_t)t * ldp;
+    const float p = (float)pos[t];
+    const int half = r / 2;
+    // queries
+    for (int idx = threadIdx.x; idx < H * d; idx += blockDim.x) {
+        const int h = idx / d, c = idx - h * d;
+        q_plain[(size_t)t * H * d + idx] = tl_from_float<T>(row[h * (d + r) + c]);
+    }
+    for (int idx = threadIdx.x; idx < H * (D - rank); idx += blockDim.x) {
+        const int h = idx / (D - rank), c = idx - h * (D - rank);
+        float v = 0.f;
+        if (c < r) {
+            const int i = c < half ? c : c - half;
+            const float a = p * freq[i];
+            const float cs = cosf(a) * mag, sn = sinf(a) * mag;
+            const float* qr = row + h * (d + r) + d;
+            v = c < half ? qr[i] * cs - qr[i + half] * sn : qr[i + half] * cs + qr[i] * sn;
+        }
+        q_lat[((size_t)t * H + h) * D + rank + c] = tl_from_float<T>(v);
+    }
+    // the latent and the shared rotated key part
+    const float* kv = row + H * (d + r);
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < rank; c += blockDim.x) ss += kv[c] * kv[c];
+    ss = tl_block_sum(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)rank + eps);
+    const int slot = slots[t];
+    if (slot < 0) return;
+    const size_t pg = (size_t)slot / page, within = (size_t)slot % page;
+    for (int c = threadIdx.x; c < D; c += blockDim.x) {
+        float v = 0.f;
+        if (c < rank) {
+            v = kv[c] * rstd * norm_w[c];
+        } else if (c < rank + r) {
+            const int cc = c - rank;
+            const int i = cc < half ? cc : cc - half;
+            const float a = p * freq[i];
+            const float cs = cosf(a) * mag, sn = sinf(a) * mag;
+            const float* kr = kv + rank;
+            v = cc < half ? kr[i] * cs - kr[i + half] * sn : kr[i + half] * cs + kr[i] * sn;
+        }
+        const T o = tl_from_float<T>(v);
+        k_cache[(size_t)slot * D + c] = o;
+        v_cache[(pg * D + c) * page + within] = o;
+    }
+}
+
+extern "C" int tl_latent_prepare(const float* proj, int ldp, const int32_t* pos, const float* freq, float mag,
+                                 const float* norm_w, float eps, const int32_t* slots, void* q_plain, void* q_lat,
+                                 void* k_cache, void* v_cache, int dtype, int T, int H, int d, int r, int rank, int D, int page,
+                                 hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && H > 0 && d > 0 && r >= 0 && r % 2 == 0 && rank > 0 && D >= rank + r && page > 0,
+                 "tl_latent_prepare: bad sizes H=%d d=%d r=%d rank=%d D=%d", H, d, r, rank, D);
+    TL_CHECK_ARG(ldp >= H * (d + r) + rank + r, "tl_latent_prepare: the projection's rows are too short");
+    if (T == 0) return 0;
+    dim3 grid(T), block(256);
+    if (dtype == TL_F32)
+        hipLaunchKernelGGL(latent_prepare_kernel<float>, grid, block, 0, stream, proj, ldp, pos, freq, mag, norm_w, eps, slots,
+                           (float*)q_plain, (float*)q_lat, (float*)k_cache, (float*)v_cache, H, d, r, rank, D, page);
+    else if (dtype == TL_BF16)
+        hipLaunchKernelGGL(latent_prepare_kernel<bf16_t>, grid, block, 0, stream, proj, ldp, pos, freq, mag, norm_w, eps, slots,
+                           (bf16_t*)q_plain, (bf16_t*)q_lat, (bf16_t*)k_cache, (bf16_t*)v_cache, H, d, r, rank, D, page);
+    else return tl_fail("tl_latent_prepare: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_latent_prepare");
+    return 0;
+}
+
+// ---- a gate per head ---------------------------------------------------------------------------------------
+// o [T, H*dv] *= sigmoid(gate[t, h]) (gate float with row stride ldg), in place.
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ o, const float* __restrict__ gate, int ldg, int H, int dv) {
+    const int t = blockIdx.x;
+    for (int idx = threadIdx.x; idx < H * dv; idx += blockDim.x) {
+        const int h = idx / dv;
+        const size_t at = (size_t)t * H * dv + idx;
+        o[at] = tl_from_float<T>(tl_to_float(o[at]) * pw_sigmoid(gate[(size_t)t * ldg + h]));
+    }
+}
+
+extern "C" int tl_head_gate(void* o, int dtype, const float* gate, int ldg, int T, int H, int dv, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && H > 0 && dv > 0 && ldg >= H, "tl_head_gate: bad sizes");
+    if (T == 0) return 0;
+    dim3 grid(T), block(256);
+    if (dtype == TL_F32) hipLaunchKernelGGL(head_gate_kernel<float>, grid, block, 0, stream, (float*)o, gate, ldg, H, dv);
+    else if (dtype == TL_BF16) hipLaunchKernelGGL(head_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)o, gate, ldg, H, dv);
+    else return tl_fail("tl_head_gate: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_head_gate");
+    return 0;
+}

@@ -59,6 +59,22 @@ class DecoderModel:
         return fn(self.embedding) if fn is not None else {}
 
     def load_tensors(self, get: Callable[[str], torch.Tensor]) -> None:
+        # a tensor that several parts declare (one table that every layer reads a slice of) is
+        # fetched once and shared
+        counts: dict[str, int] = {}
+        for p in self._all_parts():
+            for name in p.tensors():
+                counts[name] = counts.get(name, 0) + 1
+        shared: dict[str, torch.Tensor] = {}
+        fetch = get
+
+        def get(name: str) -> torch.Tensor:
+            if counts.get(name, 0) <= 1:
+                return fetch(name)
+            if name not in shared:
+                shared[name] = fetch(name)
+            return shared[name]
+
         self.embedding.load(get)
         for b in self.blocks:
             for p in b.parts():

@@ -890,3 +890,276 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     _call("tl_sample", _ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature), _ptr(top_p),
           _ptr(uniform), _ptr(out), _ptr(pmax), _ptr(ws), 1 if any_greedy else 0, 1 if any_top_p else 0, _stream())
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# Norms without statistics, gated and grouped norms, token shift, per-layer token input
+def _f32(t: torch.Tensor, what: str, n: int | None = None) -> None:
+    _check(t.dtype == torch.float32 and t.is_contiguous(), f"{what} must be a contiguous float32 tensor")
+    if n is not None:
+        _check(t.numel() == n, f"{what} has {t.numel()} entries, {n} are needed")
+
+
+def add_dyt(x: torch.Tensor, residual: torch.Tensor | None, weight: torch.Tensor, bias: torch.Tensor, alpha: torch.Tensor,
+            out_dtype: torch.dtype, rows: torch.Tensor | None = None) -> torch.Tensor:
+    """Dynamic Tanh in place of a norm: without ``rows``, ``x += residual`` in place (float32) and
+    ``tanh(alpha x) * weight + bias`` is returned; with ``rows`` the same of ``x[rows] +
+    residual[rows]`` with ``x`` left alone.  ``alpha`` is a one-element float32 tensor on the device."""
+    _on_gpu(x, residual, weight, bias, alpha, rows)
+    _check(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "add_dyt: x must be contiguous float32 [T, H]")
+    T, H = x.shape
+    _f32(weight, "add_dyt weight", H)
+    _f32(bias, "add_dyt bias", H)
+    _f32(alpha, "add_dyt alpha", 1)
+    res_code = F32
+    if residual is not None:
+        _check(residual.is_contiguous() and tuple(residual.shape) == (T, H), "add_dyt: residual must match x")
+        res_code = _code(residual, "add_dyt residual")
+    n = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.numel()
+    out = torch.empty(n, H, dtype=out_dtype, device=x.device)
+    _call("tl_add_dyt", _ptr(x), _ptr(residual), res_code, _ptr(weight), _ptr(bias), _ptr(alpha), _ptr(out),
+          _code(out, "add_dyt out"), _ptr(rows), n, H, _stream())
+    return out
+
+
+def add_cast(x: torch.Tensor, residual: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor:
+    """``x += residual`` in place (both float32) and ``x`` again in ``out_dtype``."""
+    _on_gpu(x, residual)
+    _check(x.dtype == torch.float32 and x.is_contiguous(), "add_cast: x must be contiguous float32")
+    if residual is not None:
+        _check(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape == x.shape,
+               "add_cast: the residual must be float32 of x's shape")
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _call("tl_add_cast", _ptr(x), _ptr(residual), _ptr(out), _code(out, "add_cast out"), ctypes.c_longlong(x.numel()), _stream())
+    return out
+
+
+def tanh_rows(z: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """``tanh(z)`` of a float32 tensor, in ``out_dtype``."""
+    _on_gpu(z)
+    _check(z.dtype == torch.float32 and z.is_contiguous(), "tanh_rows: input must be contiguous float32")
+    out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+    _call("tl_unary", _ptr(z), _ptr(out), _code(out, "tanh_rows out"), ctypes.c_longlong(z.numel()), 0, _stream())
+    return out
+
+
+def clamp_glu(gate_up: torch.Tensor, limit: float, alpha: float, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """For a fused [T, 2F] projection (gate columns first): ``g = min(gate, limit)``, ``u = clamp(up,
+    -limit, limit)``, result ``g * sigmoid(alpha g) * (u + 1)`` [T, F]."""
+    _on_gpu(gate_up)
+    _check(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "clamp_glu: input must be contiguous [T, 2F]")
+    T, F2 = gate_up.shape
+    out = torch.empty(T, F2 // 2, dtype=out_dtype or gate_up.dtype, device=gate_up.device)
+    _call("tl_clamp_glu", _ptr(gate_up), _code(gate_up, "clamp_glu in"), _ptr(out), _code(out, "clamp_glu out"), T, F2 // 2,
+          ctypes.c_float(limit), ctypes.c_float(alpha), _stream())
+    return out
+
+
+def gated_group_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, group: int, eps: float, gate_act: str,
+                     out_dtype: torch.dtype) -> torch.Tensor:
+    """``o`` float32 [T, N] in groups of ``group`` columns, each divided by its root mean square (eps
+    inside the root), times ``weight`` [N], times ``sigmoid(gate)`` or ``silu(gate)`` (``gate`` float32
+    [T, N], rows may be strided)."""
+    _on_gpu(o, weight, gate)
+    T, N = o.shape
+    _check(o.dtype == torch.float32 and o.stride(1) == 1 and gate.dtype == torch.float32 and gate.stride(1) == 1
+           and tuple(gate.shape) == (T, N), "gated_group_norm: o and gate must be float32 [T, N]")
+    _f32(weight, "gated_group_norm weight", N)
+    _check(gate_act in ("sigmoid", "silu") and group > 0 and N % group == 0, "gated_group_norm: bad group or gate")
+    out = torch.empty(T, N, dtype=out_dtype, device=o.device)
+    _call("tl_gated_group_norm", _ptr(o), o.stride(0) if T > 1 else N, _ptr(weight), _ptr(gate), gate.stride(0) if T > 1 else N,
+          _ptr(out), _code(out, "gated_group_norm out"), T, N, int(group), ctypes.c_float(eps), 0 if gate_act == "sigmoid" else 1,
+          _stream())
+    return out
+
+
+def _state_ptr(state: torch.Tensor, offset: int) -> tuple[ctypes.c_void_p, int]:
+    """(address of element ``offset`` of slot 0, elements from one slot to the next) of a float32
+    state arena [slots, n]."""
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous() and 0 <= offset < state.shape[1],
+           "a state arena must be contiguous float32 [slots, n]")
+    return ctypes.c_void_p(state.data_ptr() + 4 * offset), state.shape[1]
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, ctx, state: torch.Tensor, offset: int) -> torch.Tensor:
+    """``out[m, t] = h[t] + (before[t] - h[t]) * mu[m]`` for each mixing vector ``mu[m]`` (float32
+    [ways, W]), where ``before[t]`` is the row above in the same sequence, and for a sequence's first
+    row of the step the row its state slot keeps at ``state[slot, offset : offset + W]`` (zeros for a new
+    request).  Afterwards each sequence's last row of the step is kept there."""
+    _on_gpu(h, mu, state)
+    T, W = h.shape
+    _check(h.is_contiguous() and mu.dim() == 2 and mu.shape[1] == W, "token_shift: bad shapes")
+    _f32(mu, "token_shift mu")
+    _check(offset + W <= state.shape[1], "token_shift: the kept row does not fit the state")
+    prev, stride = _state_ptr(state, offset)
+    out = torch.empty(mu.shape[0], T, W, dtype=h.dtype, device=h.device)
+    _call("tl_token_shift", _ptr(h), _code(h, "token_shift"), _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(ctx.state_slots),
+          prev, ctypes.c_longlong(stride), _ptr(mu), _ptr(out), T, ctx.num_seqs, W, mu.shape[0], _stream())
+    return out
+
+
+def gelu_token_gate(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0: int) -> torch.Tensor:
+    """``gelu_tanh(z[t]) * table[ids[t], col0 : col0 + D]`` for float32 ``z`` [T, D], in the table's dtype."""
+    _on_gpu(z, table, ids)
+    T, D = z.shape
+    _f32(z, "gelu_token_gate input")
+    _i32(ids, "ids", T)
+    _check(table.dim() == 2 and table.is_contiguous() and col0 + D <= table.shape[1], "gelu_token_gate: bad table")
+    out = torch.empty(T, D, dtype=table.dtype, device=z.device)
+    _call("tl_gelu_token_gate", _ptr(z), _ptr(table), _code(table, "gelu_token_gate table"), _ptr(ids), _ptr(out), T, D,
+          table.shape[1], int(col0), table.shape[0], _stream())
+    return out
+
+
+def latent_prepare(proj: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor, mag: float, norm_weight: torch.Tensor, eps: float,
+                   slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, heads: int, dim: int, rot: int,
+                   rank: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """What a latent-attention step does between its projections and the attention kernel.  ``proj``
+    float32 [T, >= heads * (dim + rot) + rank + rot]: the query heads (plain part, then the part to
+    rotate), the compressed row and the rotated key part all heads share.  The compressed row is RMS
+    normed (``norm_weight``, ``eps``), the rotated parts are turned (pair i with i + rot/2, angle
+    ``pos * freq[i]``, cosine and sine times ``mag``), and the row [latent | rotated key | zeros] of D =
+    the cache's width goes into both cache planes at ``slots``.  Returns (plain query parts [T, heads *
+    dim], queries in the latent space [T, heads * D] with only the columns from ``rank`` on filled in),
+    both in the cache's dtype."""
+    _on_gpu(proj, pos, freq, norm_weight, slots, k_cache, v_cache)
+    T = proj.shape[0]
+    D, page = k_cache.shape[3], k_cache.shape[1]
+    _check(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "latent_prepare: the projection must be float32 [T, n]")
+    _check_caches(k_cache, v_cache, k_cache.dtype, 1, D, "latent_prepare")
+    _check(D >= rank + rot and 2 * freq.numel() == rot, "latent_prepare: sizes do not fit the cache")
+    _f32(freq, "latent_prepare freq")
+    _f32(norm_weight, "latent_prepare norm weight", rank)
+    _i32(pos, "pos", T)
+    _i32(slots, "slots", T)
+    q_plain = torch.empty(T, heads * dim, dtype=k_cache.dtype, device=proj.device)
+    q_lat = torch.empty(T, heads * D, dtype=k_cache.dtype, device=proj.device)
+    _call("tl_latent_prepare", _ptr(proj), proj.stride(0) if T > 1 else proj.shape[1], _ptr(pos), _ptr(freq), ctypes.c_float(mag),
+          _ptr(norm_weight), ctypes.c_float(eps), _ptr(slots), _ptr(q_plain), _ptr(q_lat), _ptr(k_cache), _ptr(v_cache),
+          _code(k_cache, "latent_prepare cache"), T, heads, dim, rot, rank, D, page, _stream())
+    return q_plain, q_lat
+
+
+def head_gate(o: torch.Tensor, gate: torch.Tensor, heads: int) -> torch.Tensor:
+    """``o`` [T, heads * dv], in place: head h times ``sigmoid(gate[t, h])`` (``gate`` float32, rows may be strided)."""
+    _on_gpu(o, gate)
+    T = o.shape[0]
+    _check(o.is_contiguous() and o.shape[1] % heads == 0 and gate.dtype == torch.float32 and gate.stride(1) == 1
+           and tuple(gate.shape) == (T, heads), "head_gate: bad shapes")
+    _call("tl_head_gate", _ptr(o), _code(o, "head_gate"), _ptr(gate), gate.stride(0) if T > 1 else heads, T, heads,
+          o.shape[1] // heads, _stream())
+    return o
+
+
+def batched_linear(a: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """A product per head in one launch: ``out[:, b] = a[:, b] @ weights[b].T`` for ``a`` [T, B, K],
+    ``weights`` [B, N, K] contiguous and ``out`` [T, B, N]; ``a`` and ``out`` may be views into wider rows
+    (unit stride along K and N, any stride along T and B)."""
+    _on_gpu(a, weights, out)
+    T, B, K = a.shape
+    N = weights.shape[1]
+    _check(weights.is_contiguous() and tuple(weights.shape) == (B, N, K) and tuple(out.shape) == (T, B, N)
+           and a.stride(2) == 1 and out.stride(2) == 1 and a.dtype == weights.dtype == out.dtype, "batched_linear: bad shapes")
+    if T == 0:
+        return out
+    _call("tl_gemm_generic_batched", _ptr(a), _code(a, "batched_linear"), _ptr(weights), _code(weights, "batched_linear"),
+          _ptr(out), _code(out, "batched_linear"), T, N, K, a.stride(0) if T > 1 else max(K, a.stride(0)),
+          out.stride(0) if T > 1 else max(N, out.stride(0)), B, ctypes.c_longlong(a.stride(1)),
+          ctypes.c_longlong(N * K), ctypes.c_longlong(out.stride(1)), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# Recurrences over a matrix state per head
+def recurrence_takes_key_dim(dk: int) -> bool:
+    return bool(library().tl_linear_recurrence_takes(int(dk)))
+
+
+def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ctx, state: torch.Tensor, heads: int, dk: int,
+                      dv: int, decay: torch.Tensor | None = None, wlog: torch.Tensor | None = None,
+                      bonus: torch.Tensor | None = None, silu_inputs: bool = False) -> torch.Tensor:
+    """Per sequence and head, token by token, with the state S [dk, dv] of the sequence's slot
+    (``state[slot, : heads * dk * dv]``, float32, updated in place):
+
+    * ``decay`` float32 [heads]: ``S <- decay_h S + k_t v_t^T``, ``o_t = S^T q_t``;
+    * ``wlog`` float32 [T, heads * dk] and ``bonus`` [heads, dk]: ``o_t = (S + diag(bonus) k_t v_t^T)^T
+      q_t``, then ``S <- diag(exp(-exp(wlog_t))) S + k_t v_t^T``.
+
+    ``q``, ``k`` [T, heads * dk] and ``v`` [T, heads * dv] are float32 and may be column blocks of a
+    wider matrix; ``silu_inputs`` applies SiLU to all three on the way in.  Returns float32 [T, heads * dv]."""
+    _on_gpu(q, k, v, state, decay, wlog, bonus)
+    T = q.shape[0]
+    for name, t, n in (("q", q, heads * dk), ("k", k, heads * dk), ("v", v, heads * dv)):
+        _check(t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1 and tuple(t.shape) == (T, n),
+               f"linear_recurrence: {name} must be float32 [T, {n}]")
+    per_token = wlog is not None
+    if per_token:
+        _check(wlog.dtype == torch.float32 and wlog.stride(1) == 1 and tuple(wlog.shape) == (T, heads * dk), "linear_recurrence: bad decays")
+        if bonus is not None:
+            _f32(bonus, "linear_recurrence bonus", heads * dk)
+    else:
+        _check(decay is not None, "linear_recurrence: a decay per head or per token is needed")
+        _f32(decay, "linear_recurrence decay", heads)
+    _check(heads * dk * dv <= state.shape[1], "linear_recurrence: the state of a request is too small")
+    st, stride = _state_ptr(state, 0)
+    out = torch.empty(T, heads * dv, dtype=torch.float32, device=q.device)
+    ld = lambda t: t.stride(0) if T > 1 else max(t.shape[1], t.stride(0))
+    _call("tl_linear_recurrence", _ptr(q), ld(q), _ptr(k), ld(k), _ptr(v), ld(v), _ptr(wlog), ld(wlog) if per_token else 0,
+          _ptr(decay), _ptr(bonus), 1 if per_token else 0, st, ctypes.c_longlong(stride), _ptr(ctx.state_slots),
+          _ptr(ctx.q_start), _ptr(out), heads * dv, ctx.num_seqs, heads, dk, dv, 1 if silu_inputs else 0, _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# Routed experts
+def moe_route(logits: torch.Tensor, top: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per row of float32 ``logits`` [T, E]: the ``top`` largest (lowest index first among equals), as
+    int32 ids [T, top], and the softmax over those alone, float32 [T, top]."""
+    _on_gpu(logits)
+    T, E = logits.shape
+    _check(logits.dtype == torch.float32 and logits.stride(1) == 1, "moe_route: logits must be float32 [T, E]")
+    ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    weights = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    _call("tl_moe_route", _ptr(logits), logits.stride(0) if T > 1 else E, _ptr(ids), _ptr(weights), T, E, int(top), _stream())
+    return ids, weights
+
+
+def moe_tile_rows(pairs: int, experts: int) -> int:
+    """Rows of a tile of the grouped products: 16 where an expert gets few pairs (decode steps), else 64."""
+    return 16 if pairs <= 16 * experts else 64
+
+
+def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+                limit: float, alpha: float, shared: torch.Tensor | None = None) -> torch.Tensor:
+    """``out[t] = sum_c weights[t, c] * expert_{ids[t, c]}(h[t]) (+ shared[t])`` in float32, where expert
+    e is ``down[e] @ act(gate_up[e] @ h)`` with the clamped gated activation of :func:`clamp_glu`.
+    ``gate_up`` [E, 2F, K] (gate rows first), ``down`` [E, N, F]; ``h`` [T, K] in the weights' dtype."""
+    _on_gpu(h, gate_up, down, ids, weights, shared)
+    T, K = h.shape
+    E, F2, _ = gate_up.shape
+    F, N, top = F2 // 2, down.shape[1], ids.shape[1]
+    _check(h.stride(1) == 1 and gate_up.is_contiguous() and down.is_contiguous() and gate_up.shape[2] == K
+           and tuple(down.shape) == (E, N, F) and h.dtype == gate_up.dtype == down.dtype, "moe_experts: bad shapes")
+    _check(ids.dtype == torch.int32 and ids.is_contiguous() and tuple(ids.shape) == (T, top), "moe_experts: bad ids")
+    _f32(weights, "moe_experts weights", T * top)
+    if shared is not None:
+        _f32(shared, "moe_experts shared", T * N)
+    P = T * top
+    BM = moe_tile_rows(P, E)
+    max_tiles = P // BM + E
+    order = torch.empty(P, dtype=torch.int32, device=h.device)
+    tiles = torch.empty(1 + 3 * max_tiles, dtype=torch.int32, device=h.device)
+    _call("tl_moe_sort", _ptr(ids), _ptr(order), _ptr(tiles), P, E, BM, _stream())
+    act = torch.empty(P, F, dtype=h.dtype, device=h.device)
+    _call("tl_moe_gemm", _ptr(h), _code(h, "moe_experts input"), h.stride(0) if T > 1 else K, _ptr(gate_up),
+          _code(gate_up, "moe_experts weights"), _ptr(act), _code(act, "moe_experts"), F, _ptr(order), _ptr(tiles), max_tiles, BM,
+          top, F, K, 1, ctypes.c_float(limit), ctypes.c_float(alpha), _stream())
+    y = torch.empty(P, N, dtype=torch.float32, device=h.device)
+    _call("tl_moe_gemm", _ptr(act), _code(act, "moe_experts"), F, _ptr(down), _code(down, "moe_experts weights"), _ptr(y), F32, N,
+          _ptr(order), _ptr(tiles), max_tiles, BM, top, N, F, 0, ctypes.c_float(0.0), ctypes.c_float(0.0), _stream())
+    out = torch.empty(T, N, dtype=torch.float32, device=h.device)
+    _call("tl_moe_combine", _ptr(y), _ptr(weights), _ptr(shared), _ptr(out), T, N, top, _stream())
+    return out

@@ -57,8 +57,13 @@ class Part:
 class Linear:
     """``y = x W^T + b`` with W [out, in] as checkpoints store it (reference: tensorline/quant.py:3)."""
 
-    def __init__(self, name: str, in_features: int, out_features: int, bias: bool, std: float = 0.02):
+    def __init__(self, name: str, in_features: int, out_features: int, bias: bool, std: float = 0.02,
+                 weight_name: str | None = None, bias_name: str | None = None):
+        """``weight_name`` / ``bias_name``: the tensors' checkpoint names where they are not
+        ``name + ".weight"`` / ``name + ".bias"``."""
         self.name = name
+        self.weight_name = weight_name or name + ".weight"
+        self.bias_name = bias_name or name + ".bias"
         self.in_features, self.out_features, self.has_bias, self.std = in_features, out_features, bias, std
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
@@ -66,14 +71,14 @@ class Linear:
         self.shuffled_float: torch.Tensor | None = None   # the same for a float32 weight (the 32-bit path's decode steps)
 
     def tensors(self) -> dict[str, TensorDecl]:
-        out = {self.name + ".weight": TensorDecl((self.out_features, self.in_features), "normal", self.std, "compute")}
+        out = {self.weight_name: TensorDecl((self.out_features, self.in_features), "normal", self.std, "compute")}
         if self.has_bias:
-            out[self.name + ".bias"] = TensorDecl((self.out_features,), "normal", self.std, "float32")
+            out[self.bias_name] = TensorDecl((self.out_features,), "normal", self.std, "float32")
         return out
 
     def load(self, get: TensorGetter) -> None:
-        self.weight = get(self.name + ".weight")
-        self.bias = get(self.name + ".bias") if self.has_bias else None
+        self.weight = get(self.weight_name)
+        self.bias = get(self.bias_name) if self.has_bias else None
 
     def prepare(self) -> "Linear":
         """Make the second, matrix-core ordered copy of a bfloat16 weight.  Decode steps stream

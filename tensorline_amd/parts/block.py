@@ -97,3 +97,47 @@ class PreNormBlock:
 def _deferrable(norm):
     fn = getattr(norm, "deferrable", None)
     return fn() if fn is not None else None
+
+
+@register_block("prenorm_token_input")
+class PreNormTokenInputBlock:
+    """Pre-norm order with two things the plain block does not have: the feed-forward (and its norm)
+    may be absent, and a per-layer input from the token ids may follow it:
+
+        x <- x + carry;  x <- x + mixer(norm1(x));  [x <- x + ffn(norm2(x))];  [carry = token_input(x)]
+
+    What the last stage leaves is handed on, not added: the next block's first norm (or the final
+    norm) adds it in its own pass.  Carries are plain float32 tensors; no norm rides on a product
+    here, so any norm kind fits."""
+
+    def __init__(self, spec: LayerSpec, hidden_size: int, dtype, device):
+        common = dict(hidden_size=hidden_size, dtype=dtype, device=device)
+        self.spec = spec
+        self.mixer_norm = build_part("norm", spec.mixer_norm, layer_prefix=spec.prefix, **common)
+        self.mixer = build_part("mixer", spec.mixer, layer_prefix=spec.prefix, **common)
+        self.feed_forward_norm = self.feed_forward = self.token_input = None
+        if spec.feed_forward is not None:
+            self.feed_forward_norm = build_part("norm", spec.feed_forward_norm, layer_prefix=spec.prefix, **common)
+            self.feed_forward = build_part("feed_forward", spec.feed_forward, layer_prefix=spec.prefix, **common)
+        if spec.token_input is not None:
+            self.token_input = build_part("token_input", spec.token_input, layer_prefix=spec.prefix, **common)
+
+    def parts(self) -> list[Part]:
+        return [p for p in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward, self.token_input)
+                if p is not None]
+
+    def cache_need(self):
+        fn = getattr(self.mixer, "cache_need", None)
+        return fn() if fn is not None else None
+
+    def state_need(self):
+        fn = getattr(self.mixer, "state_need", None)
+        return fn() if fn is not None else None
+
+    def forward(self, x: torch.Tensor, carry, ctx, cache):
+        y = self.mixer.forward(self.mixer_norm.forward(x, carry), ctx, cache)
+        if self.feed_forward is not None:
+            y = self.feed_forward.forward(self.feed_forward_norm.forward(x, y), ctx)
+        if self.token_input is not None:
+            y = self.token_input.forward(x, y, ctx)
+        return y

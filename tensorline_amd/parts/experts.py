@@ -1,0 +1,90 @@
+"""Routed experts: a feed-forward of many small gated layers of which every token uses a few.
+
+    z = W_router h + b  (float32);  the ``top`` experts with the largest z, weights = softmax over
+    those ``top`` logits alone;  out = sum_chosen weight_e * expert_e(h)  (+ shared(h))
+    expert(h) = W_down (g * sigmoid(alpha g) * (u + 1)),  g = min(W_gate h, limit),  u = clamp(W_up h, +-limit)
+
+The experts' matrices are stacked ([experts, 2 ff, width] gate over up, [experts, width, ff]); a
+step's (token, choice) pairs are ordered by expert on the device and both products run as one
+grouped launch each (``kernels.moe_experts``), with no look at the device from the host, so the
+step can be captured in a graph.  The shared expert, which every token uses, is a plain dense
+feed-forward of the same form on the framework's ordinary products.
+"""
+from __future__ import annotations
+
+import torch
+
+from tensorline_amd.ops import kernels
+from tensorline_amd.parts.base import Linear, Part, TensorGetter, fuse_linears
+from tensorline_amd.parts.registry import register_feed_forward
+from tensorline_amd.parts.spec import TensorDecl
+
+
+@register_feed_forward("routed_experts")
+class RoutedExperts(Part):
+    """Parameters: ``experts``, ``top``, ``ff`` and ``limit`` of an expert, ``shared`` = {ff, limit} or
+    None, ``alpha`` of the gate's sigmoid.  Tensors under the prefix: router, router.b, e<i>.gate /
+    .up / .down, shared.gate / .up / .down."""
+
+    def __init__(self, hidden_size, prefix, dtype, device, experts: int, top: int, ff: int, limit: float,
+                 shared: dict | None = None, alpha: float = 1.702):
+        super().__init__(hidden_size, prefix, dtype, device)
+        self.experts, self.top, self.ff, self.limit, self.alpha = int(experts), int(top), int(ff), float(limit), float(alpha)
+        if not 0 < self.top <= self.experts or self.top > 32 or self.experts > 1024:
+            raise ValueError(f"{prefix}: top {self.top} of {self.experts} experts is not served (top <= 32, experts <= 1024)")
+        self.router = Linear(prefix + "router", hidden_size, self.experts, True, weight_name=prefix + "router",
+                             bias_name=prefix + "router.b")
+        self.gate_up = self.down = None
+        self.shared_ff = int(shared["ff"]) if shared else 0
+        self.shared_limit = float(shared["limit"]) if shared else 0.0
+        self._sg = self._su = self.shared_gate_up = self.shared_down = None
+        if shared:
+            p = prefix + "shared."
+            self._sg = Linear(p + "gate", hidden_size, self.shared_ff, False, weight_name=p + "gate")
+            self._su = Linear(p + "up", hidden_size, self.shared_ff, False, weight_name=p + "up")
+            self.shared_down = Linear(p + "down", self.shared_ff, hidden_size, False, weight_name=p + "down")
+
+    def tensors(self):
+        out = dict(self.router.tensors())
+        for e in range(self.experts):
+            p = f"{self.prefix}e{e}."
+            out[p + "gate"] = TensorDecl((self.ff, self.hidden_size), "normal", 0.05, "compute")
+            out[p + "up"] = TensorDecl((self.ff, self.hidden_size), "normal", 0.05, "compute")
+            out[p + "down"] = TensorDecl((self.hidden_size, self.ff), "normal", 0.05, "compute")
+        if self.shared_down is not None:
+            for lin in (self._sg, self._su, self.shared_down):
+                out.update(lin.tensors())
+        return out
+
+    def load(self, get: TensorGetter) -> None:
+        self.router.load(get)
+        self.router.prepare()
+        name = lambda e, s: f"{self.prefix}e{e}.{s}"
+        self.gate_up = torch.stack([torch.cat([get(name(e, "gate")), get(name(e, "up"))]) for e in range(self.experts)]).contiguous()
+        self.down = torch.stack([get(name(e, "down")) for e in range(self.experts)]).contiguous()
+        if self.shared_down is not None:
+            self._sg.load(get)
+            self._su.load(get)
+            self.shared_gate_up = fuse_linears(self.prefix + "shared.gate_up", [self._sg, self._su])
+            self._sg.weight = self._su.weight = None
+            self.shared_down.load(get)
+            self.shared_down.prepare()
+
+    def weight_tensors(self):
+        out = self.router.tensors_kept() + [self.gate_up, self.down]
+        if self.shared_down is not None:
+            out += self.shared_gate_up.tensors_kept() + self.shared_down.tensors_kept()
+        return out
+
+    def library_products(self):
+        if self.shared_down is None:
+            return []
+        return [(self.shared_gate_up.weight, self.dtype), (self.shared_down.weight, torch.float32)]
+
+    def forward(self, h, ctx):
+        ids, weights = kernels.moe_route(self.router(h, out_dtype=torch.float32), self.top)
+        shared = None
+        if self.shared_down is not None:
+            act = kernels.clamp_glu(self.shared_gate_up(h, out_dtype=torch.float32), self.shared_limit, self.alpha, self.dtype)
+            shared = self.shared_down(act, out_dtype=torch.float32)
+        return kernels.moe_experts(h, self.gate_up, self.down, ids, weights, self.limit, self.alpha, shared)

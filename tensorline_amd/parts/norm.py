@@ -1,4 +1,4 @@
-"""RMSNorm, fused with the residual add that precedes it.
+"""Norms, fused with the residual add that precedes them: RMSNorm and Dynamic Tanh.
 
 ``h = forward(x, residual)`` does ``x += residual`` on the float32 residual stream (in place)
 and returns ``x / sqrt(mean(x^2) + eps) * weight`` in the activation dtype.  Sum of squares,
@@ -39,3 +39,32 @@ class RMSNorm(Part):
 
     def forward(self, x: torch.Tensor, residual=None, rows: torch.Tensor | None = None) -> torch.Tensor:
         return kernels.add_rmsnorm(x, residual, self.weight, self.eps, self.dtype, rows=rows)
+
+
+@register_norm("dyt")
+class DynamicTanh(Part):
+    """Dynamic Tanh in the place of a norm: ``tanh(alpha * x) * weight + bias`` with a learned scalar
+    ``alpha``; no mean or variance of the row is taken.  Tensors: ``name`` (weight), ``name + ".b"``,
+    ``name + ".alpha"`` (a scalar).  Same interface as the RMS norm: adds ``residual`` into the float32
+    stream first, in place, or works on ``rows`` only.  It cannot be carried by the products around
+    it (it is not one factor per row), so it offers no ``deferrable``."""
+
+    def __init__(self, hidden_size, prefix, dtype, device, name: str):
+        super().__init__(hidden_size, prefix, dtype, device)
+        self.name = prefix + name
+        self.weight = self.bias = self.alpha = None
+
+    def tensors(self):
+        return {self.name: TensorDecl((self.hidden_size,), "one_plus_normal", 0.1, "float32"),
+                self.name + ".b": TensorDecl((self.hidden_size,), "normal", 0.1, "float32"),
+                self.name + ".alpha": TensorDecl((), "one_plus_normal", 0.2, "float32")}
+
+    def load(self, get: TensorGetter) -> None:
+        self.weight, self.bias = get(self.name), get(self.name + ".b")
+        self.alpha = get(self.name + ".alpha").reshape(1).contiguous()
+
+    def weight_tensors(self):
+        return [self.weight, self.bias, self.alpha]
+
+    def forward(self, x: torch.Tensor, residual=None, rows: torch.Tensor | None = None) -> torch.Tensor:
+        return kernels.add_dyt(x, residual, self.weight, self.bias, self.alpha, self.dtype, rows=rows)

@@ -16,9 +16,10 @@ POSITIONS: dict[str, type] = {}
 BLOCKS: dict[str, type] = {}
 EMBEDDINGS: dict[str, type] = {}
 HEADS: dict[str, type] = {}
+TOKEN_INPUTS: dict[str, type] = {}
 
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "position": POSITIONS, "block": BLOCKS,
-           "embedding": EMBEDDINGS, "head": HEADS}
+           "embedding": EMBEDDINGS, "head": HEADS, "token_input": TOKEN_INPUTS}
 
 
 def _register(table: dict[str, type], what: str, kind: str, replace: bool) -> Callable[[type], type]:
@@ -58,6 +59,10 @@ def register_head(kind: str, replace: bool = False):
     return _register(HEADS, "head", kind, replace)
 
 
+def register_token_input(kind: str, replace: bool = False):
+    return _register(TOKEN_INPUTS, "token input", kind, replace)
+
+
 def build_part(what: str, spec: PartSpec, layer_prefix: str | None = None, **common):
     """Instantiate the part ``spec`` names: ``cls(**common, **spec.params)``; parts that read
     checkpoint tensors get ``prefix = layer_prefix + spec.prefix``."""
@@ -79,3 +84,7 @@ def _ensure_builtin() -> None:
     import tensorline_amd.parts.feedforward  # noqa: F401
     import tensorline_amd.parts.norm  # noqa: F401
     import tensorline_amd.parts.rotary  # noqa: F401
+    import tensorline_amd.parts.latent_attention  # noqa: F401
+    import tensorline_amd.parts.recurrent  # noqa: F401
+    import tensorline_amd.parts.experts  # noqa: F401
+    import tensorline_amd.parts.token_input  # noqa: F401

@@ -61,3 +61,28 @@ class NoPosition:
     def apply_and_store(self, qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots, bias=None) -> None:
         if k_cache is not None or bias is not None:
             kernels.rope_store(qkv, pos, None, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots, bias)
+
+
+def yarn_frequencies(dims: int, base: float, scaling: dict | None) -> tuple[torch.Tensor, float]:
+    """Rotation frequencies of ``dims / 2`` pairs with YaRN scaling, as float32 (computed in float64
+    and rounded once), and the factor that multiplies cosine and sine.
+
+    f_i = base^(-2i / dims).  With ``scaling`` = {factor, original, fast, slow}: the pair index at
+    which a wave completes ``t`` turns over ``original`` positions is n(t) = dims ln(original / (2 pi
+    t)) / (2 ln base); between lo = max(floor(n(fast)), 0) and hi = min(ceil(n(slow)), dims - 1) the
+    ramp r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) blends the frequency from f_i (fast pairs,
+    kept) to f_i / factor (slow pairs, stretched): f_i (1 - r_i) + f_i / factor r_i.  Cosine and sine
+    are multiplied by 0.1 ln(factor) + 1.  (YaRN: Peng, Quesnelle, Fan, Shippole, "YaRN: Efficient
+    Context Window Extension of Large Language Models".)"""
+    import math
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+    if not scaling:
+        return f.to(torch.float32), 1.0
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+    turns_at = lambda t: dims * math.log(original / (2.0 * math.pi * float(t))) / (2.0 * math.log(float(base)))
+    lo = max(math.floor(turns_at(scaling["fast"])), 0)
+    hi = min(math.ceil(turns_at(scaling["slow"])), dims - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    f = f / factor * ramp + f * (1.0 - ramp)
+    return f.to(torch.float32), 0.1 * math.log(factor) + 1.0

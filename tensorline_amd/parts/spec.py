@@ -44,10 +44,11 @@ class TensorDecl:
 class LayerSpec:
     prefix: str                       # checkpoint prefix of the layer, e.g. "model.layers.3."
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: PartSpec | None     # None: a layer without feed-forward (blocks that allow it)
     mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
-    block: str = "prenorm"            # the arrangement of the four parts
+    feed_forward_norm: PartSpec | None
+    block: str = "prenorm"            # the arrangement of the parts
+    token_input: PartSpec | None = None   # a per-layer input from the token ids, for blocks that take one
 
 
 @dataclass(frozen=True)
@@ -149,6 +150,8 @@ def keys_and_values(num_kv_heads: int, head_dim: int, window: int = 0) -> CacheN
 
 @dataclass(frozen=True)
 class StateNeed:
-    """What a mixer keeps per request, of fixed size: a tensor of ``shape`` and ``dtype``."""
+    """What a mixer keeps per request, of fixed size: a tensor of ``shape`` and ``dtype``.  A mixer
+    that keeps several things (a matrix state and the previous token's input, say) asks for one flat
+    tensor and knows the offsets of its pieces."""
     shape: tuple[int, ...]
     dtype: str = "float32"

@@ -72,6 +72,20 @@ def checkpoint_files(model_dir: str) -> dict[str, str]:
     return names
 
 
+def checkpoint_shapes(model_dir: str) -> dict[str, tuple[int, ...]]:
+    """Tensor name -> shape, from the files' headers only."""
+    from safetensors import safe_open
+    by_file: dict[str, list[str]] = {}
+    for name, path in checkpoint_files(model_dir).items():
+        by_file.setdefault(path, []).append(name)
+    shapes: dict[str, tuple[int, ...]] = {}
+    for path, names in by_file.items():
+        with safe_open(path, framework="pt") as f:
+            for name in names:
+                shapes[name] = tuple(f.get_slice(name).get_shape())
+    return shapes
+
+
 def _target_dtype(decl: TensorDecl, compute: torch.dtype) -> torch.dtype:
     if decl.storage == "compute":
         return compute
