@@ -135,14 +135,19 @@ def clamped_expert(h, w, p, limit: float):
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w[p + "down"].T
 
 
-def routed_experts(h, w, p, mlp: dict):
+def routed_experts(h, w, p, mlp: dict, margins: list | None = None):
     """The ``top`` experts with the largest router logits, weighted by the softmax over those logits
-    alone, plus the shared expert if there is one."""
+    alone, plus the shared expert if there is one.  ``margins`` receives, per token, by how much the
+    last chosen logit leads the first one left out, over the largest logit's size (a close call, which
+    rounding can turn, shows as a small number)."""
     E, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
     z = h.to(torch.float32) @ w[p + "router"].to(torch.float32).T + w[p + "router.b"].to(torch.float32)
     if h.dtype == torch.float64:
         z = h @ w[p + "router"].T + w[p + "router.b"]
     val, idx = torch.topk(z, top, dim=-1)
+    if margins is not None and top < E:
+        nxt = torch.topk(z, top + 1, dim=-1).values[:, -1]
+        margins.append((val[:, -1] - nxt) / z.abs().max(-1).values)
     weight = torch.softmax(val, dim=-1).to(h.dtype)
     out = torch.zeros_like(h)
     for e in range(E):
@@ -165,9 +170,9 @@ def token_side_input(x, tokens, w, layer: int, dim: int, eps: float):
 
 
 # ---- the whole model ---------------------------------------------------------------------------------
-def forward(tokens, w, cfg: dict, per_layer: list | None = None):
+def forward(tokens, w, cfg: dict, per_layer: list | None = None, margins: list | None = None):
     """Logits [T, vocab] of one sequence from its first token.  ``per_layer``: a list that receives
-    the residual stream after every layer."""
+    the residual stream after every layer; ``margins``: see ``routed_experts``, one entry per routed layer."""
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     eps = float(cfg["norm"]["eps"])
     side = cfg.get("token_side")
@@ -186,7 +191,7 @@ def forward(tokens, w, cfg: dict, per_layer: list | None = None):
             raise ValueError(kind)
         x = x + y
         if layer.get("mlp"):
-            x = x + routed_experts(dynamic_tanh(x, w, p + "norm2"), w, p + "mlp.", layer["mlp"])
+            x = x + routed_experts(dynamic_tanh(x, w, p + "norm2"), w, p + "mlp.", layer["mlp"], margins)
         if side:
             x = token_side_input(x, tokens, w, i, int(side["dim"]), eps)
         if per_layer is not None:

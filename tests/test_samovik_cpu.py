@@ -1,0 +1,160 @@
+"""Samovik on the CPU: the configuration reader, the model's declarations, and pins of the plain
+implementation (its recurrent mixers token by token against whole sequences, its rotation and
+its routing against closed forms)."""
+import copy
+import json
+import math
+
+import pytest
+import torch
+
+from tensorline_amd.config.model_config import ConfigError
+from tensorline_amd.config.registry import architecture_name, get_architecture, load_model_config
+from tensorline_amd.config.samovik_config import SamovikConfig
+from tensorline_amd.models.decoder import DecoderModel
+from tensorline_amd.parts.rotary import yarn_frequencies
+from tensorline_amd.parts.spec import StateNeed
+from tensorline_amd.weights.random_init import random_tensor, write_random_model
+from tests import plain_samovik as P
+from tests.samovik_helpers import CFG_A, CFG_B, CFG_C, CONFIGS, typed
+
+
+def _weights(cfg, seed=0, dtype=torch.float64):
+    model = DecoderModel(get_architecture("Samovik").build_spec(typed(cfg)), torch.float32, "cpu")
+    return {n: random_tensor(n, d, seed, "cpu").to(dtype) for n, d in model.tensor_decls().items()}
+
+
+def test_architecture_is_found_by_either_key():
+    assert architecture_name({"architecture": "Samovik"}) == "Samovik"
+    assert architecture_name({"architectures": ["Qwen2ForCausalLM"], "architecture": "x"}) == "Qwen2ForCausalLM"
+    with pytest.raises(ConfigError):
+        architecture_name({})
+    assert get_architecture("Samovik").config_cls is SamovikConfig
+
+
+def test_config_round_trip_and_errors():
+    cfg = typed(CFG_A)
+    assert cfg.hidden_size == 96 and cfg.vocab_size == 320 and cfg.num_hidden_layers == 4 and cfg.token_side_dim == 8
+    assert SamovikConfig.from_dict(cfg.to_dict()).to_dict() == cfg.to_dict()
+    assert typed(CFG_B).token_side_dim == 0
+    for breaker, text in (
+            (lambda d: d["layers"][0].__setitem__("type", "conv"), "unknown"),
+            (lambda d: d["layers"][1]["mixer"].pop("kv_rank"), "kv_rank"),
+            (lambda d: d["layers"][2]["mixer"].__setitem__("decay", [0.5]), "one entry per head"),
+            (lambda d: d["layers"][1]["mlp"]["router"].__setitem__("top", 9), "exceeds"),
+            (lambda d: d["layers"][1]["mixer"]["rot"].__setitem__("dims", 6), "rot_dim"),
+            (lambda d: d.pop("norm"), "norm.eps"),
+            (lambda d: d.__setitem__("width", 0), "width")):
+        bad = copy.deepcopy(CFG_A)
+        breaker(bad)
+        with pytest.raises(ConfigError, match=text):
+            SamovikConfig.from_dict(bad)
+
+
+def test_spec_parts_caches_and_states():
+    spec = get_architecture("Samovik").build_spec(typed(CFG_A))
+    assert [l.mixer.kind for l in spec.layers] == ["wkv", "latent_attention", "lightning_attention", "latent_attention"]
+    assert spec.layers[2].feed_forward is None and spec.layers[2].feed_forward_norm is None
+    assert all(l.token_input is not None and l.token_input.params["index"] == i for i, l in enumerate(spec.layers))
+    model = DecoderModel(spec, torch.float32, "cpu")
+    needs, states = model.cache_needs(), model.state_needs()
+    # a cached row: latent and rotated key part, rounded up to the kernels' step of 16
+    assert needs[0] is None and needs[2] is None
+    assert needs[1].planes[0].shape == (1, 64) and needs[3].planes[0].shape == (1, 80) and needs[1].window == 0
+    assert states[0] == StateNeed((3 * 16 * 16 + 96,), "float32") and states[2] == StateNeed((2 * 24 * 48,), "float32")
+    assert states[1] is None
+    decls = model.tensor_decls()
+    assert decls["side.embed"].shape == (320, 4 * 8) and decls["l0.norm1.alpha"].shape == ()
+    assert "l2.norm2" not in decls and "l2.mlp.router" not in decls and "l3.mlp.shared.gate" not in decls
+    assert decls["l0.mix.w1"].shape == (8, 96) and decls["l0.mix.w0"].shape == (48,) and decls["l1.mix.dkv"].shape == (56, 96)
+    no_side = DecoderModel(get_architecture("Samovik").build_spec(typed(CFG_B)), torch.float32, "cpu").tensor_decls()
+    assert not any(n.startswith("side.") or ".side." in n for n in no_side)
+
+
+def test_size_left_to_a_tensors_shape_is_read_from_the_checkpoint(tmp_path):
+    out = write_random_model(typed(CFG_C), str(tmp_path / "m"), seed=1)
+    raw = json.load(open(out + "/config.json"))
+    assert raw["layers"][1]["mixer"].pop("decay_rank") == 4
+    json.dump(raw, open(out + "/config.json", "w"))
+    arch, cfg = load_model_config(out)
+    assert arch.name == "Samovik" and cfg.layers[1]["mixer"]["decay_rank"] == 4
+    with pytest.raises(ValueError, match="decay_rank"):
+        arch.build_spec(SamovikConfig.from_dict(raw))
+
+
+def test_yarn_frequencies_against_their_definition():
+    f, m = yarn_frequencies(8, 100.0, None)
+    assert m == 1.0 and torch.allclose(f.double(), torch.tensor([100.0 ** (-2 * i / 8) for i in range(4)]).double(), rtol=1e-7)
+    sc = {"factor": 8.0, "original": 128, "fast": 8.0, "slow": 0.5}
+    f, m = yarn_frequencies(32, 10000.0, sc)
+    plain, mp = P.yarn_frequencies({"dims": 32, "base": 10000.0, "scaling": sc})
+    assert m == pytest.approx(0.1 * math.log(8.0) + 1.0) and m == pytest.approx(mp)
+    assert torch.allclose(f.double(), plain, rtol=1e-7)
+    base = torch.tensor([10000.0 ** (-2 * i / 32) for i in range(16)]).double()
+    ratio = f.double() / base
+    assert ratio[0] == pytest.approx(1.0) and ratio[-1] == pytest.approx(1 / 8.0)      # fast pairs kept, slow ones stretched
+    assert (ratio[1:] <= ratio[:-1] + 1e-9).all()
+
+
+def test_plain_rotation_pairs_dimension_i_with_i_plus_half():
+    x = torch.zeros(1, 1, 6, dtype=torch.float64)
+    x[0, 0, 1] = 1.0                                  # first half, pair 1; partner is dimension 3; dimension 4, 5 pass
+    x[0, 0, 5] = 7.0
+    y = P.rotate(x, torch.tensor([3]), {"dims": 4, "base": 10.0, "scaling": None})
+    a = 3 * 10.0 ** (-2 * 1 / 4)
+    assert y[0, 0].tolist() == pytest.approx([0, math.cos(a), 0, math.sin(a), 0, 7.0])
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_plain_recurrent_mixers_token_by_token_equal_whole(name):
+    cfg = CONFIGS[name]
+    w = _weights(cfg)
+    torch.manual_seed(0)
+    for i, layer in enumerate(cfg["layers"]):
+        if layer["type"] == "latent_attention":
+            continue
+        fn = P.lightning if layer["type"] == "lightning" else P.wkv
+        h = torch.randn(11, cfg["width"], dtype=torch.float64)
+        whole, end = fn(h, w, f"l{i}.mix.", layer["mixer"], 1e-6)
+        state, rows = None, []
+        for cut in ((0, 1), (1, 5), (5, 6), (6, 11)):
+            y, state = fn(h[cut[0]:cut[1]], w, f"l{i}.mix.", layer["mixer"], 1e-6, state)
+            rows.append(y)
+        assert torch.allclose(torch.cat(rows), whole, rtol=1e-10, atol=1e-12)
+        a, b = (end, state) if layer["type"] == "lightning" else (end[0], state[0])
+        assert torch.allclose(a, b, rtol=1e-10, atol=1e-12)
+
+
+def test_plain_lightning_closed_form():
+    """o_t = sum_{s<=t} decay^(t-s) (q_t . k_s) v_s."""
+    cfg = CFG_C
+    w = _weights(cfg)
+    m = cfg["layers"][0]["mixer"]
+    h = torch.randn(7, cfg["width"], dtype=torch.float64)
+    silu = torch.nn.functional.silu
+    q = silu(h @ w["l0.mix.q"].T).view(7, 2, 72)
+    k = silu(h @ w["l0.mix.k"].T).view(7, 2, 72)
+    v = silu(h @ w["l0.mix.v"].T).view(7, 2, 16)
+    o = torch.zeros(7, 2, 16, dtype=torch.float64)
+    for t in range(7):
+        for s in range(t + 1):
+            for hd in range(2):
+                o[t, hd] += m["decay"][hd] ** (t - s) * (q[t, hd] @ k[s, hd]) * v[s, hd]
+    o = o.reshape(7, 32)
+    want = (P.rms_divide(o, 1e-6) * w["l0.mix.norm"] * torch.sigmoid(h @ w["l0.mix.g"].T)) @ w["l0.mix.o"].T
+    got, _ = P.lightning(h, w, "l0.mix.", m, 1e-6)
+    assert torch.allclose(got, want, rtol=1e-9, atol=1e-12)
+
+
+def test_plain_routing_weights_and_clamps():
+    w = {"r.router": torch.tensor([[1.0], [3.0], [2.0], [-5.0]], dtype=torch.float64), "r.router.b": torch.zeros(4, dtype=torch.float64)}
+    for e in range(4):
+        w[f"r.e{e}.gate"] = torch.full((1, 1), float(e + 1), dtype=torch.float64)
+        w[f"r.e{e}.up"] = torch.full((1, 1), 10.0, dtype=torch.float64)
+        w[f"r.e{e}.down"] = torch.ones(1, 1, dtype=torch.float64)
+    mlp = {"router": {"experts": 4, "top": 2}, "expert": {"ff": 1, "limit": 2.5}, "shared": None}
+    out = P.routed_experts(torch.ones(1, 1, dtype=torch.float64), w, "r.", mlp)
+    # experts 1 and 2 (logits 3 and 2) with weights softmax(3, 2); gates 2 and 3 -> min(., 2.5); up 10 -> 2.5
+    p = math.exp(3) / (math.exp(3) + math.exp(2))
+    act = lambda g: g / (1 + math.exp(-1.702 * g)) * (2.5 + 1)
+    assert out.item() == pytest.approx(p * act(2.0) + (1 - p) * act(2.5))
