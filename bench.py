@@ -402,6 +402,132 @@ def bench_workload(args) -> int:
     return 0
 
 
+
+# ---- the hybrid design (Samovik) beside the dense decoder at equal size ------------------------------
+# Layer sizes that resemble real models of the kind: width, heads of 128, a latent of 192 + 64 rotated
+# dimensions (a cached row of 256), state mixers with heads of 128 and 64, experts of which 6 are used
+# and a shared one.  ``dense`` is the closest existing model at equal size: the same width, layers and
+# vocabulary, grouped-query attention with the same number of heads of 128, and a feed-forward as wide as
+# the experts a token uses plus the shared one.
+HYBRID_SIZES = {
+    "w1024": dict(width=1024, heads=8, experts=32, top=6, ff=512, shared_ff=1024, side=128),
+    "w2048": dict(width=2048, heads=16, experts=64, top=6, ff=1408, shared_ff=2816, side=256),
+    "w4096": dict(width=4096, heads=32, experts=64, top=6, ff=2048, shared_ff=4096, side=256),
+}
+HYBRID_VOCAB = 32000
+
+
+def make_hybrid_config(size: str):
+    from tensorline_amd.config import SamovikConfig
+    z = HYBRID_SIZES[size]
+    H = z["heads"]
+    mlp = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"]}, "expert": {"ff": z["ff"], "limit": 7.0},
+           "shared": {"ff": z["shared_ff"], "limit": 7.0}}
+    latent = {"heads": H, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5,
+              "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    lightning = {"heads": H, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** (-5 - 3 * h / H) for h in range(H)]}
+    wkv = {"heads": 2 * H, "dim": 64, "decay_rank": 64}
+    layers = [{"type": t, "mixer": m, "mlp": mlp} for t, m in
+              (("latent_attention", latent), ("lightning", lightning), ("wkv", wkv), ("latent_attention", latent))]
+    return SamovikConfig.from_dict({"architecture": "Samovik", "vocab": HYBRID_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+                                    "token_side": {"dim": z["side"]}, "layers": layers})
+
+
+def make_dense_twin(size: str):
+    from tensorline_amd.config import Qwen2Config
+    z = HYBRID_SIZES[size]
+    return Qwen2Config.from_dict(dict(
+        architectures=["Qwen2ForCausalLM"], vocab_size=HYBRID_VOCAB, hidden_size=z["width"],
+        intermediate_size=z["top"] * z["ff"] + z["shared_ff"], num_hidden_layers=4, num_attention_heads=z["heads"],
+        num_key_value_heads=max(1, z["heads"] // 4), head_dim=128, rope_theta=10000.0, rms_norm_eps=1e-6,
+        tie_word_embeddings=False, max_position_embeddings=32768))
+
+
+def profile_step(llm, entries_of, seed: int) -> dict:
+    """Event time of every kernel of one eager step, summed per entry point (milliseconds), after a
+    warm-up step of the same shape."""
+    from tensorline_amd.engine.runner import ModelRunner
+    from tensorline_amd.ops.profile import KernelTimer
+    cache = llm.cache
+    runner = ModelRunner(llm.model, cache)
+    runner.fit_context = llm.engine.runner.fit_context
+    out = {}
+    for rep in range(2):
+        entries = entries_of(cache, rep)
+        timer = KernelTimer()
+        if rep:
+            with timer.measuring():
+                runner.step(entries)
+        else:
+            runner.step(entries)
+        sync()
+        for e in entries:
+            cache.release(e.rid)
+        if rep:
+            by_name: dict = {}
+            for _, name, e0, e1 in timer._spans:
+                by_name[name] = by_name.get(name, 0.0) + e0.elapsed_time(e1)
+            out = {n: round(v, 4) for n, v in sorted(by_name.items(), key=lambda kv: -kv[1])}
+    return out
+
+
+def bench_hybrid(args) -> int:
+    """Prefill and decode throughput of the hybrid design at HYBRID_SIZES beside the dense decoder at
+    equal size, and each step's time by kernel.  One JSON line; the default benchmark is not run."""
+    import torch
+
+    from tensorline_amd import LLM
+    from tensorline_amd.engine.batch import StepEntry
+    page, tokens, batch, context = 16, args.prefill_tokens, args.batch, min(args.context, 2048)
+    sizes = [s for s in (args.hybrid_sizes.split(",") if args.hybrid_sizes else sorted(HYBRID_SIZES))]
+    results = {}
+    for size in sizes:
+        row = {}
+        for which, cfg in (("hybrid", make_hybrid_config(size)), ("dense", make_dense_twin(size))):
+            max_len = max(context, tokens) + 16
+            llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
+                      num_blocks=(batch + 1) * (-(-max_len // page)) + 8, max_num_seqs=batch, max_batched_tokens=max(2048, tokens),
+                      max_model_len=max_len, graphs=not args.no_graphs, graph_warmup_tokens=0, prefix_caching=False,
+                      tune_library=False, overlap=not args.no_overlap)
+            pre = bench_prefill(llm, tokens, 3, args.seed + 2)
+            dec = bench_decode(llm, batch, context, args.steps, args.warmup, args.seed + 1)
+            entry = {"prefill_tok_s": round(pre["tok_s"], 1), "prefill_ms": round(pre["s"] * 1e3, 3),
+                     "decode_tok_s": round(dec["tok_s"], 1), "decode_ms_per_step": round(dec["ms_per_step"], 4),
+                     "weight_GB": round(llm.model.weight_bytes() / 1e9, 3)}
+            if args.profile:
+                prompt = random_prompts(1, tokens, cfg.vocab_size, args.seed + 3)[0]
+
+                def prefill_entries(cache, rep):
+                    rid = ("pp", rep)
+                    cache.add_request(rid)
+                    assert cache.grow(rid, tokens)
+                    return [StepEntry(rid, prompt, 0, [tokens - 1])]
+
+                def decode_entries(cache, rep):
+                    out = []
+                    for b in range(batch):
+                        rid = ("pd", rep, b)
+                        cache.add_request(rid)
+                        assert cache.grow(rid, context)
+                        out.append(StepEntry(rid, [prompt[b]], context - 1, [0]))
+                    return out
+                entry["prefill_kernels_ms"] = profile_step(llm, prefill_entries, args.seed)
+                entry["decode_kernels_ms"] = profile_step(llm, decode_entries, args.seed)
+            row[which] = entry
+            del llm
+            gc.collect()
+            torch.cuda.empty_cache()
+        row["hybrid_over_dense"] = {"prefill": round(row["hybrid"]["prefill_tok_s"] / row["dense"]["prefill_tok_s"], 3),
+                                    "decode": round(row["hybrid"]["decode_tok_s"] / row["dense"]["decode_tok_s"], 3)}
+        results[size] = row
+    print(json.dumps({"metric": "hybrid_design_tok_s", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
+                      "config": {"model": "Samovik layer sizes (4 layers: latent attention, lightning, wkv, latent attention) beside "
+                                          "Qwen2 layers of equal width (4 layers)", "prefill_tokens": tokens, "decode_batch": batch,
+                                 "decode_context": context, "sizes": {k: HYBRID_SIZES[k] for k in sizes}},
+                      "results": results}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -431,12 +557,18 @@ def main() -> int:
     ap.add_argument("--output-tokens", type=int, default=512)
     ap.add_argument("--temperature", type=float, default=0.7)
     ap.add_argument("--num-blocks", type=int, default=0, help="KV pages for --workload (0: 80%% of free memory)")
+    ap.add_argument("--hybrid", action="store_true",
+                    help="instead of the default benchmark: the hybrid design (Samovik) at real layer sizes beside the dense "
+                         "decoder at equal size, prefill and decode; with --profile each step's time by kernel")
+    ap.add_argument("--hybrid-sizes", default="", help="which of w1024,w2048,w4096 (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
     if args.workload:
         return bench_workload(args)
+    if args.hybrid:
+        return bench_hybrid(args)
 
     import torch
 

@@ -23,46 +23,59 @@
 #define MOE_MAX_TOP 32
 
 // ---- routing ------------------------------------------------------------------------------------------
-__global__ void moe_route_kernel(const float* __restrict__ logits, int ldl, int32_t* __restrict__ ids,
-                                 float* __restrict__ weights, int T, int E, int top) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+// A wave per token: lane l looks at logits l, l + 64, ...; the largest not yet chosen is found by a
+// butterfly over (value, index), equal values going to the lower index; lane c keeps the c-th choice.
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ldl, int32_t* __restrict__ ids,
+                                                        float* __restrict__ weights, int T, int E, int top) {
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (t >= T) return;
     const float* z = logits + (size_t)t * ldl;
-    int chosen[MOE_MAX_TOP];
-    float val[MOE_MAX_TOP];
+    const int none = 0x7fffffff;
+    unsigned taken = 0;                 // bit s: logit lane + 64 s is chosen already
+    float my_val = 0.f;
+    int my_id = 0;
     for (int c = 0; c < top; ++c) {
-        int best = -1;
         float bv = 0.f;
-        for (int e = 0; e < E; ++e) {
-            bool taken = false;
-            for (int p = 0; p < c; ++p) taken |= chosen[p] == e;
-            if (taken) continue;
+        int be = none;
+        for (int e = lane, sl = 0; e < E; e += 64, ++sl) {
+            if ((taken >> sl) & 1u) continue;
             const float v = z[e];
-            if (best < 0 || v > bv || (v != v && bv == bv)) {      // a NaN logit is chosen, so that it shows
-                best = e;
+            if (be == none || v > bv) {
                 bv = v;
+                be = e;
             }
         }
-        chosen[c] = best;
-        val[c] = bv;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oe = __shfl_xor(be, off, 64);
+            if (oe != none && (be == none || ov > bv || (ov == bv && oe < be))) {
+                bv = ov;
+                be = oe;
+            }
+        }
+        if ((be & 63) == lane) taken |= 1u << (be >> 6);
+        if (lane == c) {
+            my_val = bv;
+            my_id = be;
+        }
     }
-    float sum = 0.f;
-    const float largest = val[0];
-    for (int c = 0; c < top; ++c) {
-        val[c] = expf(val[c] - largest);
-        sum += val[c];
-    }
-    for (int c = 0; c < top; ++c) {
-        ids[(size_t)t * top + c] = chosen[c];
-        weights[(size_t)t * top + c] = val[c] / sum;
+    const float largest = __shfl(my_val, 0, 64);
+    const float ex = lane < top ? expf(my_val - largest) : 0.f;
+    const float sum = tl_wave_sum(ex);
+    if (lane < top) {
+        ids[(size_t)t * top + lane] = my_id;
+        weights[(size_t)t * top + lane] = ex / sum;
     }
 }
 
 extern "C" int tl_moe_route(const float* logits, int ldl, int32_t* ids, float* weights, int T, int E, int top,
                             hipStream_t stream) {
-    TL_CHECK_ARG(T >= 0 && E > 0 && top > 0 && top <= E && top <= MOE_MAX_TOP && ldl >= E, "tl_moe_route: bad sizes E=%d top=%d", E, top);
+    TL_CHECK_ARG(T >= 0 && E > 0 && top > 0 && top <= E && top <= MOE_MAX_TOP && E <= MOE_MAX_EXPERTS && ldl >= E,
+                 "tl_moe_route: bad sizes E=%d top=%d", E, top);
     if (T == 0) return 0;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(tl_ceil_div(T, 64)), dim3(64), 0, stream, logits, ldl, ids, weights, T, E, top);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(tl_ceil_div(T, 4)), dim3(256), 0, stream, logits, ldl, ids, weights, T, E, top);
     TL_CHECK_LAUNCH("tl_moe_route");
     return 0;
 }
@@ -264,6 +277,123 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_kernel(const TA* __restri
     }
 }
 
+// The same product for bfloat16 operands on v_mfma_f32_16x16x32_bf16 (products exact, sums in float).
+// Tiles of BM x 128 matrix rows per work-group (GLU: 64 gate rows and the 64 up rows of the same
+// columns), k in steps of 64 through double-buffered LDS whose rows are padded to 144 bytes, so that the
+// sixteen 16-byte fragment reads of a quarter wave fall into different banks; the next step's pieces
+// wait in registers meanwhile.  Lane l = 16 g + c gives row c of a block at the eight k from 8 g on,
+// as first operand (a row of A) and as second (a row of W), and holds C[4 g + v][c] in register v.
+typedef __bf16 mg_bf16x8 __attribute__((ext_vector_type(8)));
+#define MGB_KT 64
+#define MGB_LD 72
+
+template <int MB, bool GLU>
+__global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda,
+                                                                  const bf16_t* __restrict__ W, void* __restrict__ Cv, int ldc,
+                                                                  const int32_t* __restrict__ order,
+                                                                  const int32_t* __restrict__ tiles, int top, int N, int K,
+                                                                  float limit, float alpha) {
+    constexpr int BM = MB * 16, WR = 128, BN = GLU ? 64 : 128;
+    constexpr int A_PIECES = BM * 8, W_PIECES = WR * 8;
+    constexpr int A_PER = (A_PIECES + MG_THREADS - 1) / MG_THREADS, W_PER = W_PIECES / MG_THREADS;
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * MGB_LD];
+    __shared__ __attribute__((aligned(16))) uint16_t Ws[2][WR * MGB_LD];
+    __shared__ int arow[BM];
+    if ((int)blockIdx.y >= tiles[0]) return;
+    const int e = tiles[1 + 3 * blockIdx.y], place0 = tiles[2 + 3 * blockIdx.y], rows = tiles[3 + 3 * blockIdx.y];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * BN;
+    for (int r = tid; r < BM; r += MG_THREADS) arow[r] = r < rows ? (GLU ? order[place0 + r] / top : place0 + r) : -1;
+    __syncthreads();
+    const bf16_t* We = W + (size_t)e * (GLU ? 2 : 1) * N * K;
+
+    mg_f32x4 acc[MB][2];
+#pragma unroll
+    for (int i = 0; i < MB; ++i) acc[i][0] = acc[i][1] = (mg_f32x4){0.f, 0.f, 0.f, 0.f};
+
+    uint4 areg[A_PER], wreg[W_PER];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int it = 0; it < A_PER; ++it) {
+            const int p = tid + it * MG_THREADS;
+            const int r = p >> 3, k = k0 + 8 * (p & 7);
+            const int src = p < A_PIECES ? arow[r] : -1;
+            areg[it] = (src >= 0 && k < K) ? *reinterpret_cast<const uint4*>(A + (size_t)src * lda + k) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int it = 0; it < W_PER; ++it) {
+            const int p = tid + it * MG_THREADS;
+            const int r = p >> 3, k = k0 + 8 * (p & 7);
+            const int col = (GLU && r >= 64) ? n0 + r - 64 : n0 + r;
+            const size_t wrow = (GLU && r >= 64) ? (size_t)N + col : (size_t)col;
+            wreg[it] = (col < N && k < K) ? *reinterpret_cast<const uint4*>(We + wrow * K + k) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto to_lds = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < A_PER; ++it) {
+            const int p = tid + it * MG_THREADS;
+            if (p < A_PIECES) *reinterpret_cast<uint4*>(&As[buf][(p >> 3) * MGB_LD + 8 * (p & 7)]) = areg[it];
+        }
+#pragma unroll
+        for (int it = 0; it < W_PER; ++it) {
+            const int p = tid + it * MG_THREADS;
+            *reinterpret_cast<uint4*>(&Ws[buf][(p >> 3) * MGB_LD + 8 * (p & 7)]) = wreg[it];
+        }
+    };
+    // W rows of this wave's two blocks: GLU gate block `wave` and up block `wave`; else blocks 2 wave, 2 wave + 1
+    const int wr0 = (GLU ? wave * 16 : wave * 32) + c, wr1 = (GLU ? 64 + wave * 16 : wave * 32 + 16) + c;
+
+    fetch(0);
+    to_lds(0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += MGB_KT) {
+        const bool more = k0 + MGB_KT < K;
+        if (more) fetch(k0 + MGB_KT);
+#pragma unroll
+        for (int s = 0; s < MGB_KT / 32; ++s) {
+            const mg_bf16x8 w0 = __builtin_bit_cast(mg_bf16x8, *reinterpret_cast<const uint4*>(&Ws[buf][wr0 * MGB_LD + 32 * s + 8 * g]));
+            const mg_bf16x8 w1 = __builtin_bit_cast(mg_bf16x8, *reinterpret_cast<const uint4*>(&Ws[buf][wr1 * MGB_LD + 32 * s + 8 * g]));
+#pragma unroll
+            for (int i = 0; i < MB; ++i) {
+                const mg_bf16x8 a = __builtin_bit_cast(mg_bf16x8, *reinterpret_cast<const uint4*>(&As[buf][(i * 16 + c) * MGB_LD + 32 * s + 8 * g]));
+                acc[i][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, w0, acc[i][0], 0, 0, 0);
+                acc[i][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, w1, acc[i][1], 0, 0, 0);
+            }
+        }
+        if (more) {
+            to_lds(buf ^ 1);
+            __syncthreads();
+            buf ^= 1;
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int r = i * 16 + 4 * g + v;
+            if (r >= rows) continue;
+            if (GLU) {
+                const int n = n0 + wave * 16 + c;
+                if (n >= N) continue;
+                const float gt = fminf(acc[i][0][v], limit);
+                const float up = fminf(fmaxf(acc[i][1][v], -limit), limit);
+                reinterpret_cast<bf16_t*>(Cv)[(size_t)(place0 + r) * ldc + n] =
+                    tl_from_float<bf16_t>(gt * (1.0f / (1.0f + expf(-alpha * gt))) * (up + 1.0f));
+            } else {
+                float* crow = reinterpret_cast<float*>(Cv) + (size_t)order[place0 + r] * ldc;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int n = n0 + wave * 32 + j * 16 + c;
+                    if (n < N) crow[n] = acc[i][j][v];
+                }
+            }
+        }
+}
+
 // glu 1: A [T, K] tokens (row stride lda), W [E, 2N, K], C [P, N] by place, of type c_dtype.
 // glu 0: A [P, K] by place, W [E, N, K], C float [P, N] by pair.  max_tiles bounds the tiles that
 // tl_moe_sort can have made: P / BM + E.
@@ -285,6 +415,22 @@ extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, i
         if (BM == 16) GO(TA, TW, TO, 1, 1, GLU); \
         else GO(TA, TW, TO, 4, 1, GLU);          \
     } while (0)
+    const bool bf = a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == (glu ? TL_BF16 : TL_F32);
+    if (bf && K % 8 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0) {
+#define GO_BF(MB, GLU)                                                                                                   \
+    hipLaunchKernelGGL((moe_gemm_bf16_kernel<MB, GLU>), dim3(tl_ceil_div(N, GLU ? 64 : 128), max_tiles), dim3(MG_THREADS), 0, \
+                       stream, (const bf16_t*)A, lda, (const bf16_t*)W, C, ldc, order, tiles, top, N, K, limit, alpha)
+        if (glu) {
+            if (BM == 16) GO_BF(1, true);
+            else GO_BF(4, true);
+        } else {
+            if (BM == 16) GO_BF(1, false);
+            else GO_BF(4, false);
+        }
+#undef GO_BF
+        TL_CHECK_LAUNCH("tl_moe_gemm");
+        return 0;
+    }
     if (glu) {
         if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32) GO_BM(float, float, float, true);
         else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_BF16) GO_BM(bf16_t, bf16_t, bf16_t, true);
