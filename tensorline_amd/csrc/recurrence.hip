@@ -14,16 +14,19 @@
 // a position are the same bits however the sequence was cut into steps and whatever else is in the
 // batch.
 //
-// A work-group of four waves owns 64 value columns of one head of one sequence.  Lane j of wave g
-// keeps S[g R .. g R + R)[j] in registers (R = ceil(dk / 4) rounded up to a template size); queries,
-// keys, decays and values of REC_TB tokens at a time go through LDS, the four waves' shares of an
-// output are added in the order of the waves.
+// A work-group of four waves owns 16 value columns of one head of one sequence: that gives a prompt
+// of one sequence heads x value columns / 16 work-groups to spread over the GPU, and what a token
+// costs is the length of one thread's chain of instructions, not arithmetic.  Lane 16 r + j of wave g
+// keeps rows (4 g + r) R .. + R of column j of S in registers (R = ceil(dk / 16) rounded up to a
+// template size); queries, keys, decays and values of 16 tokens at a time go through LDS, the next
+// chunk's on their way in registers meanwhile; a column's sixteen shares of an output are left in
+// LDS and added in ascending order of the rows once per chunk.
 #include "common.h"
 
 #include <math.h>
 
-#define REC_TB 8
 #define REC_MAX_DK 256
+#define REC_COLS 16
 
 __device__ __forceinline__ float rec_silu(float z) { return z / (1.0f + expf(-z)); }
 
@@ -33,61 +36,72 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(
     const float* __restrict__ wlog, int ldw, const float* __restrict__ decay, const float* __restrict__ bonus,
     float* __restrict__ state, long long state_stride, const int32_t* __restrict__ state_slots,
     const int32_t* __restrict__ q_start, float* __restrict__ out, int ldo, int H, int dk, int dv, int silu_inputs) {
-    __shared__ float qs[REC_TB][4 * R], ks[REC_TB][4 * R], ws[PER_TOKEN ? REC_TB : 1][4 * R], vs[REC_TB][64];
-    __shared__ float part[4][REC_TB][64];
+    constexpr int DKP = 16 * R;                       // rows the tile holds; those beyond dk stay zero
+    constexpr int REC_TB = R == 16 ? 8 : 16;          // tokens per chunk (fewer for the largest tile: LDS)
+    constexpr int PER = REC_TB * DKP / 256;           // elements of a [REC_TB][DKP] tile per thread
+    __shared__ __attribute__((aligned(16))) float qs[REC_TB][DKP], ks[REC_TB][DKP], ws[PER_TOKEN ? REC_TB : 1][DKP];
+    __shared__ float vs[REC_TB][REC_COLS];
+    __shared__ float part[16][REC_TB][REC_COLS];      // a row group's share of every output of the chunk
     const int tid = threadIdx.x, lane = tid & 63, g = tid >> 6;
-    const int j0 = blockIdx.x * 64, h = blockIdx.y, s = blockIdx.z;
+    const int col = lane & 15, rg = 4 * g + (lane >> 4);
+    const int j0 = blockIdx.x * REC_COLS, h = blockIdx.y, s = blockIdx.z;
     const int r0 = q_start[s], r1 = q_start[s + 1];
     if (r1 <= r0) return;
-    const int j = j0 + lane;
+    const int j = j0 + col;
     const bool col_ok = j < dv;
     float* st = state + (size_t)state_slots[s] * state_stride + (size_t)h * dk * dv;
 
     float S[R], ur[R];
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
-        const int i = g * R + rr;
+        const int i = rg * R + rr;
         S[rr] = (i < dk && col_ok) ? st[(size_t)i * dv + j] : 0.f;
         ur[rr] = (PER_TOKEN && bonus && i < dk) ? bonus[h * dk + i] : 1.f;
     }
     const float dec = PER_TOKEN ? 1.f : decay[h];
-    // rows of the LDS tiles beyond dk stay zero: they multiply state rows that are zero and stay zero
-    for (int idx = tid; idx < REC_TB * 4 * R; idx += 256) {
-        (&qs[0][0])[idx] = 0.f;
-        (&ks[0][0])[idx] = 0.f;
-        if (PER_TOKEN) (&ws[0][0])[idx] = 0.f;
-    }
 
+    // The next REC_TB tokens' operands are read into registers while this chunk is computed (with one
+    // work-group or less per CU nothing else would hide those reads), and go to LDS afterwards: element
+    // tid + 256 it of the [REC_TB][DKP] tile, R to a thread; what lies outside the step or the head is zero.
+    float qreg[PER], kreg[PER], wreg[PER_TOKEN ? PER : 1], vreg = 0.f;
+    auto fetch = [&](int t0, int n) {
+#pragma unroll
+        for (int it = 0; it < PER; ++it) {
+            const int idx = tid + it * 256, tt = idx / DKP, i = idx - tt * DKP;
+            const bool ok = tt < n && i < dk;
+            qreg[it] = ok ? q[(size_t)(t0 + tt) * ldq + h * dk + i] : 0.f;
+            kreg[it] = ok ? k[(size_t)(t0 + tt) * ldk + h * dk + i] : 0.f;
+            if (PER_TOKEN) wreg[it] = ok ? wlog[(size_t)(t0 + tt) * ldw + h * dk + i] : 0.f;
+        }
+        const int tt = tid / REC_COLS, jj = tid % REC_COLS;      // beyond the chunk for tid >= REC_TB * REC_COLS: tt >= n
+        vreg = (tt < n && j0 + jj < dv) ? v[(size_t)(t0 + tt) * ldv + h * dv + j0 + jj] : 0.f;
+    };
+    auto stash = [&](int n) {
+#pragma unroll
+        for (int it = 0; it < PER; ++it) {
+            const int idx = tid + it * 256, tt = idx / DKP, i = idx - tt * DKP;
+            const bool ok = tt < n && i < dk;
+            (&qs[0][0])[idx] = silu_inputs ? rec_silu(qreg[it]) : qreg[it];
+            (&ks[0][0])[idx] = silu_inputs ? rec_silu(kreg[it]) : kreg[it];
+            if (PER_TOKEN) (&ws[0][0])[idx] = ok ? expf(-expf(wreg[it])) : 0.f;
+        }
+        if (tid < REC_TB * REC_COLS) (&vs[0][0])[tid] = silu_inputs ? rec_silu(vreg) : vreg;
+    };
+
+    fetch(r0, min(REC_TB, r1 - r0));
+    stash(min(REC_TB, r1 - r0));
+    __syncthreads();
     for (int t0 = r0; t0 < r1; t0 += REC_TB) {
         const int n = min(REC_TB, r1 - t0);
-        __syncthreads();
-        for (int idx = tid; idx < n * dk; idx += 256) {
-            const int tt = idx / dk, i = idx - tt * dk;
-            float qv = q[(size_t)(t0 + tt) * ldq + h * dk + i], kv = k[(size_t)(t0 + tt) * ldk + h * dk + i];
-            if (silu_inputs) {
-                qv = rec_silu(qv);
-                kv = rec_silu(kv);
-            }
-            qs[tt][i] = qv;
-            ks[tt][i] = kv;
-            if (PER_TOKEN) ws[tt][i] = expf(-expf(wlog[(size_t)(t0 + tt) * ldw + h * dk + i]));
-        }
-        for (int idx = tid; idx < n * 64; idx += 256) {
-            const int tt = idx >> 6, jj = idx & 63;
-            float vv = 0.f;
-            if (j0 + jj < dv) {
-                vv = v[(size_t)(t0 + tt) * ldv + h * dv + j0 + jj];
-                if (silu_inputs) vv = rec_silu(vv);
-            }
-            vs[tt][jj] = vv;
-        }
-        __syncthreads();
+        const bool more = t0 + REC_TB < r1;
+        if (more) fetch(t0 + REC_TB, min(REC_TB, r1 - t0 - REC_TB));
+#pragma unroll 4
         for (int tt = 0; tt < n; ++tt) {
-            const float vj = vs[tt][lane];
+            const float vj = vs[tt][col];
             float acc = 0.f;
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
-                const int i = g * R + rr;
+                const int i = rg * R + rr;
                 const float kv = ks[tt][i] * vj;
                 if (PER_TOKEN) {
                     acc += qs[tt][i] * (S[rr] + ur[rr] * kv);
@@ -97,18 +111,24 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(
                     acc += qs[tt][i] * S[rr];
                 }
             }
-            part[g][tt][lane] = acc;
+            part[rg][tt][col] = acc;
         }
         __syncthreads();
-        for (int idx = tid; idx < n * 64; idx += 256) {
-            const int tt = idx >> 6, jj = idx & 63;
-            if (j0 + jj < dv)
-                out[(size_t)(t0 + tt) * ldo + h * dv + j0 + jj] = ((part[0][tt][jj] + part[1][tt][jj]) + part[2][tt][jj]) + part[3][tt][jj];
+        {
+            const int tt = tid / REC_COLS, jj = tid % REC_COLS;
+            if (tt < n && j0 + jj < dv) {
+                float sum = part[0][tt][jj];
+#pragma unroll
+                for (int r = 1; r < 16; ++r) sum += part[r][tt][jj];       // the row groups in ascending order
+                out[(size_t)(t0 + tt) * ldo + h * dv + j0 + jj] = sum;
+            }
         }
+        if (more) stash(min(REC_TB, r1 - t0 - REC_TB));
+        __syncthreads();
     }
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
-        const int i = g * R + rr;
+        const int i = rg * R + rr;
         if (i < dk && col_ok) st[(size_t)i * dv + j] = S[rr];
     }
 }
@@ -130,7 +150,7 @@ extern "C" int tl_linear_recurrence(const float* q, int ldq, const float* k, int
     TL_CHECK_ARG(per_token ? (wlog != nullptr && ldw >= H * dk) : decay != nullptr, "tl_linear_recurrence: decays are missing");
     TL_CHECK_ARG(H <= 65535 && S <= 65535, "tl_linear_recurrence: too many heads or sequences for one launch");
     if (S == 0) return 0;
-    dim3 grid(tl_ceil_div(dv, 64), H, S), block(256);
+    dim3 grid(tl_ceil_div(dv, REC_COLS), H, S), block(256);
 #define GO(R)                                                                                                            \
     do {                                                                                                                 \
         if (per_token)                                                                                                   \
@@ -140,11 +160,11 @@ extern "C" int tl_linear_recurrence(const float* q, int ldq, const float* k, int
             hipLaunchKernelGGL((linear_recurrence_kernel<R, false>), grid, block, 0, stream, q, ldq, k, ldk, v, ldv, wlog, ldw, \
                                decay, bonus, state, state_stride, state_slots, q_start, out, ldo, H, dk, dv, silu_inputs); \
     } while (0)
-    if (dk <= 16) GO(4);
-    else if (dk <= 32) GO(8);
-    else if (dk <= 64) GO(16);
-    else if (dk <= 128) GO(32);
-    else GO(64);
+    if (dk <= 16) GO(1);
+    else if (dk <= 32) GO(2);
+    else if (dk <= 64) GO(4);
+    else if (dk <= 128) GO(8);
+    else GO(16);
 #undef GO
     TL_CHECK_LAUNCH("tl_linear_recurrence");
     return 0;
