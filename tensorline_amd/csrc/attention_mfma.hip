@@ -850,7 +850,7 @@ __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     const int s_lo = (lo >> 5) / split_blocks, s_hi = (p >> 5) / split_blocks;
     const int ns = s_hi - s_lo + 1;
     const size_t base = ((size_t)wrow * nq + h) * nsplit + s_lo;
-    const int D4 = D >> 2, SG = AM_MERGE_THREADS / D4;      // D is 32, 64 or 128
+    const int D4 = D >> 2, SG = AM_MERGE_THREADS / D4;      // D is 32, 64, 128 or 256
     const int d4 = tid % D4, sg = tid / D4;
     const float4* acc4 = reinterpret_cast<const float4*>(ws_o) + base * D4 + d4;
     const float2* ml2 = reinterpret_cast<const float2*>(ws_ml) + base;
@@ -965,7 +965,7 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
                                  const int32_t* seq_list, int n_list, int skip_single, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_mfma: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_mfma: %d query heads are not a multiple of %d key/value heads", nq, nkv);
-    TL_CHECK_ARG(d == 32 || d == 64 || d == 128, "tl_attention_mfma: head size %d is not one of 32, 64, 128", d);
+    TL_CHECK_ARG(d == 32 || d == 64 || d == 128 || d == 256, "tl_attention_mfma: head size %d is not one of 32, 64, 128, 256", d);
     TL_CHECK_ARG(bs >= 8 && bs % 8 == 0, "tl_attention_mfma: page size %d must be a multiple of 8", bs);
     TL_CHECK_ARG(NT == 1 || NT == 2, "tl_attention_mfma: NT=%d must be 1 or 2", NT);
     TL_CHECK_ARG(nsplit >= 1 && nsplit <= AM_MAX_SPLITS && max_tile_groups >= 1,
@@ -992,7 +992,9 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     dim3 grid(S_run, nkv, (unsigned)((waves + wg_waves - 1) / wg_waves));
     const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
     const bool pow2 = (bs & (bs - 1)) == 0;
-    if (NT == 2 && nsplit == 1 && shared && pow2 && !seq_list && total_groups128 > 0 &&
+    // (a head size of 256 has the independent waves only: its tiles of keys and values would not leave
+    // LDS for a second work-group per CU)
+    if (NT == 2 && nsplit == 1 && shared && pow2 && !seq_list && total_groups128 > 0 && d != 256 &&
         at_lds_bytes(d / 32, NB, S) <= 160 * 1024) {
         // 128 columns per work-group, keys and values shared through LDS; shared == 2 asks for two
         // chains per work-group where their tiles fit LDS
@@ -1026,8 +1028,11 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     else if (d == 64)
         launch_attn<2>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
                        ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
-    else
+    else if (d == 128)
         launch_attn<4>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
+    else
+        launch_attn<8>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
                        ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
     TL_CHECK_LAUNCH("tl_attention_mfma");
     if (nsplit > 1) {

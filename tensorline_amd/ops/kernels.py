@@ -333,6 +333,7 @@ def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tenso
 
 
 MAX_KEY_SPLITS = 1024    # key splits the attention merge kernel takes
+MFMA_HEAD_DIMS = (32, 64, 128, 256)   # head sizes of the bfloat16 matrix-core attention (256: its independent-wave kernel only)
 GENERIC_SPLIT_KEYS = 256  # keys per split of the any-shape attention kernel in steps of one token per sequence
 SKINNY_MAX_ROWS = 16     # rows the few-row kernel serves (one 16-row MFMA tile)
 ROWS64_MAX_ROWS = 64     # rows the 17..64-row kernel serves; above that the library
@@ -737,7 +738,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     q_stride = q.stride(0) if T > 1 else q.shape[1]
     o_stride = out.stride(0) if T > 1 else out.shape[1]
     page = k_cache.shape[1]
-    mfma_ok = (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and page % 8 == 0 and q_start is not None
+    mfma_ok = (q.dtype == torch.bfloat16 and head_dim in MFMA_HEAD_DIMS and page % 8 == 0 and q_start is not None
                and ctx_start is not None and plan is not None and q_stride % 8 == 0 and o_stride % 4 == 0
                and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0)
     if path in ("mfma", "mfma-direct", "mfma-tile16", "mfma-tile16x2", "mfma-tile32"):
@@ -755,7 +756,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             split_len, nsplit = _key_splits(len(singles), num_kv_heads, ctx1, plan.fit_context)
             if route_singles or (route_singles is None and nsplit > 1 and _singles_get_own_launch(
                     plan, singles, num_heads, num_kv_heads, head_dim, int(window))):
-                nt1 = 1 if G <= 16 else 2
+                nt1 = 1 if G <= 16 or head_dim == 256 else 2      # a head size of 256: one column tile per wave (registers)
                 ws = torch.empty(len(singles) * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
                 n_o = len(singles) * num_heads * nsplit * head_dim
                 _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
@@ -765,7 +766,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                       _stream())
                 skip_single = 1
         q_lens = [n for n in plan.q_lens if n > 1] if skip_single else plan.q_lens
-        nt = 1 if plan.max_query_len * G <= 16 else 2
+        nt = 1 if plan.max_query_len * G <= 16 or head_dim == 256 else 2
         groups = [-(-n * G // (16 * nt)) for n in q_lens]
         pads = 0 if skip_single else max(0, S - len(groups))    # padding sequences bring one token each
         max_groups = max(groups + [1])

@@ -14,7 +14,7 @@ head's rows of W_uk, the plain part of a score is (U_h^T q_h^plain(i)) . c(j): t
 into the latent space once per token, the attention kernel then sees H query heads over ONE shared
 key/value head whose key is [c | R(k^rot)] and whose value is c, and the head's rows of W_uv are
 applied to the weighted sum of latents afterwards.  That is the paged attention the framework
-already has, with ``num_kv_heads`` 1 and a head size of kv_rank + rot_dim (rounded up to 16).
+already has, with ``num_kv_heads`` 1 and a head size of kv_rank + rot_dim (rounded up to 32, 64, 128 or 256).
 """
 from __future__ import annotations
 
@@ -43,11 +43,12 @@ class LatentAttention(Part):
         if int(rot.get("dims", self.rot_dim)) != self.rot_dim or self.rot_dim % 2:
             raise ValueError(f"{prefix}: the rotation turns {rot.get('dims')} dimensions, the rotated part has {self.rot_dim}; "
                              "they must be equal and even")
-        # the width of a cached row: latent, rotated key part, zeros up to the kernels' step of 16
-        self.cache_dim = -(-(self.rank + self.rot_dim) // 16) * 16
-        if not kernels.attention_takes_head_dim(self.cache_dim):
-            raise ValueError(f"{prefix}: kv_rank + rot_dim = {self.rank + self.rot_dim} is not served: the attention "
-                             "kernels take rows of up to 256")
+        # the width of a cached row: latent, rotated key part, zeros up to the next head size that the
+        # matrix-core attention kernels take (32, 64, 128, 256)
+        need = self.rank + self.rot_dim
+        self.cache_dim = next((d for d in kernels.MFMA_HEAD_DIMS if d >= need), 0)
+        if not self.cache_dim:
+            raise ValueError(f"{prefix}: kv_rank + rot_dim = {need} is not served: the attention kernels take rows of up to 256")
         freq, self.mag = yarn_frequencies(self.rot_dim, float(rot["base"]), rot.get("scaling"))
         self.freq = freq.to(device)
         H = self.heads

@@ -58,9 +58,9 @@ def test_spec_parts_caches_and_states():
     assert all(l.token_input is not None and l.token_input.params["index"] == i for i, l in enumerate(spec.layers))
     model = DecoderModel(spec, torch.float32, "cpu")
     needs, states = model.cache_needs(), model.state_needs()
-    # a cached row: latent and rotated key part, rounded up to the kernels' step of 16
+    # a cached row: latent and rotated key part, rounded up to a head size of the attention kernels
     assert needs[0] is None and needs[2] is None
-    assert needs[1].planes[0].shape == (1, 64) and needs[3].planes[0].shape == (1, 80) and needs[1].window == 0
+    assert needs[1].planes[0].shape == (1, 64) and needs[3].planes[0].shape == (1, 128) and needs[1].window == 0
     assert states[0] == StateNeed((3 * 16 * 16 + 96,), "float32") and states[2] == StateNeed((2 * 24 * 48,), "float32")
     assert states[1] is None
     decls = model.tensor_decls()

@@ -67,6 +67,8 @@ MIXERS = [
     ("latent_attention", _latent(3, 24, 8, 40, 48, scaling={"factor": 3.0, "original": 32, "fast": 8.0, "slow": 1.0})),
     ("latent_attention", _latent(1, 10, 6, 7, 20, base=20.0)),
     ("latent_attention", _latent(5, 16, 16, 32, 112, base=1e6, scale=0.3)),        # rows of 128: the bfloat16 matrix-core kernels
+    ("latent_attention", _latent(4, 32, 8, 16, 200, base=500.0)),                     # rows of 256
+    ("latent_attention", _latent(18, 8, 8, 8, 140)),                                  # rows of 256, more heads than a tile of 16
     ("lightning", {"heads": 2, "dim": 24, "vdim": 48, "decay": [0.9, 0.999]}),
     ("lightning", {"heads": 1, "dim": 130, "vdim": 66, "decay": [1.0]}),
     ("lightning", {"heads": 3, "dim": 7, "vdim": 5, "decay": [0.1, 0.5, 0.7]}),
@@ -81,7 +83,7 @@ def test_mixer_alone(case, dtype):
     kind, mixer = MIXERS[case]
     cfg = one_layer(kind, mixer, width=72)
     model, w = build(cfg, dtype, seed=case)
-    lens = [37, 1, 18]
+    lens = [37, 1, 150] if kind == "latent_attention" else [37, 1, 18]
     ctx, views = _context(model, [tokens_for(cfg, n, s) for s, n in enumerate(lens)])
     torch.manual_seed(case)
     h = torch.randn(sum(lens), 72).to(torch.bfloat16).float()
