@@ -338,3 +338,66 @@ def test_greedy_generation_through_the_entry_point(name, tmp_path):
         outs = llm.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0))
         assert [o.token_ids for o in outs] == want
         assert llm.cache.all_free()
+
+
+def test_command_line_random_model_generate_and_trace_program(tmp_path):
+    """The programs a user runs: ``tensorline random-model`` from a config.json, ``tensorline generate`` on the
+    folder (greedy, and sampled with a seed twice), and ``bin/trace_run`` fed steps on its standard input."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = copy.deepcopy(CFG_B)
+    (tmp_path / "cfg.json").write_text(json.dumps(cfg))
+    tl = [sys.executable, os.path.join(root, "bin", "tensorline")]
+    folder = str(tmp_path / "m")
+    proc = subprocess.run(tl + ["random-model", "--config", str(tmp_path / "cfg.json"), "--out", folder, "--seed", "4"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    # the folder's config.json may leave the decay's bottleneck width to the tensor's shape
+    raw = json.load(open(folder + "/config.json"))
+    del raw["layers"][1]["mixer"]["decay_rank"]
+    json.dump(raw, open(folder + "/config.json", "w"))
+    from safetensors import safe_open
+    w = {}
+    with safe_open(folder + "/model.safetensors", "pt") as f:
+        for k in f.keys():
+            w[k] = f.get_tensor(k).float()
+    prompts = [tokens_for(cfg, 19, 1), tokens_for(cfg, 4, 2)]
+    want = []
+    for p in prompts:
+        seq = list(p)
+        for _ in range(6):
+            seq.append(int(P.forward(seq, w, cfg)[-1].argmax()))
+        want.append(seq[len(p):])
+    base = tl + ["generate", "--model", folder, "--dtype", "float32", "--num-blocks", "32", "--block-size", "8",
+                 "--max-tokens", "6", "--stop-token-id", "-1"]
+    for p in prompts:
+        base += ["--prompt-ids", " ".join(map(str, p))]
+    proc = subprocess.run(base, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    recs = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
+    assert [r["token_ids"] for r in recs] == want
+    sampled = []
+    for _ in range(2):
+        proc = subprocess.run(base + ["--temperature", "0.9", "--top-p", "0.8", "--seed", "7"], capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        sampled.append([json.loads(l)["token_ids"] for l in proc.stdout.splitlines() if l.startswith("{")])
+    assert sampled[0] == sampled[1] and all(len(t) == 6 for t in sampled[0])
+    # the trace program: a prompt in two portions, then one token; logits at three places
+    toks = prompts[0]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:7], "want": [6]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[7:18], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": toks[18:], "want": [0]}], "end": ["a"]}]
+    out = tmp_path / "out"
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(out),
+                           "--max-tokens", "64"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    ref = P.forward(toks, w, cfg).numpy()
+    assert not (out / "1.f32").exists()
+    for step, place in ((0, 6), (2, 18)):
+        got = np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(1, -1)
+        assert rel_error(got[0], ref[place]) < LIMIT["float32"]
