@@ -9,13 +9,6 @@
 
 #include <math.h>
 
-template <typename T> __device__ __forceinline__ float pw_read(const void* p, size_t i) {
-    return tl_to_float(reinterpret_cast<const T*>(p)[i]);
-}
-template <typename T> __device__ __forceinline__ void pw_write(void* p, size_t i, float v) {
-    reinterpret_cast<T*>(p)[i] = tl_from_float<T>(v);
-}
-
 __device__ __forceinline__ float pw_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float pw_silu(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float pw_gelu_tanh(float z) {
@@ -358,5 +351,95 @@ extern "C" int tl_head_gate(void* o, int dtype, const float* gate, int ldg, int 
     else if (dtype == TL_BF16) hipLaunchKernelGGL(head_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)o, gate, ldg, H, dv);
     else return tl_fail("tl_head_gate: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("tl_head_gate");
+    return 0;
+}
+
+// ---- attention over wide rows -----------------------------------------------------------------------------
+// Causal attention of H query heads over ONE shared key/value head whose rows are wider than the
+// matrix-core kernels take (D up to 1024): the key of a cached token is its whole row of D columns, its
+// value the same row.  q [T, H*D], cache rows token-major [pages, page, 1, D], out [T, H*D]; float
+// arithmetic, no matrix instructions: the slow and simple way for sizes nothing else serves.
+// A work-group per (token, head); wave w takes the keys j with j % 4 == w (by absolute position, so the
+// same keys meet in a wave however the sequence was cut), each lane the columns lane, lane + 64, ... of
+// query, key and running sum; per key a sum over the wave, then the online softmax step.  The four waves'
+// sums are put together in the order of the waves.
+#define WIDE_MAX_D 1024
+template <typename T>
+__global__ __launch_bounds__(256) void attn_wide_kernel(const T* __restrict__ q, const T* __restrict__ kc,
+                                                        const int32_t* __restrict__ tables, int NB,
+                                                        const int32_t* __restrict__ seq_of_token,
+                                                        const int32_t* __restrict__ pos, T* __restrict__ out, int H, int D,
+                                                        int page, float scale) {
+    constexpr int E = WIDE_MAX_D / 64;
+    __shared__ float sm[4], sl[4];
+    __shared__ float sacc[4][WIDE_MAX_D];
+    const int t = blockIdx.x, h = blockIdx.y;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int s = seq_of_token[t], p = pos[t];
+    const int32_t* table = tables + (size_t)s * NB;
+    const T* qrow = q + ((size_t)t * H + h) * D;
+    float qv[E], acc[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int c = lane + 64 * e;
+        qv[e] = c < D ? tl_to_float(qrow[c]) * scale : 0.f;
+        acc[e] = 0.f;
+    }
+    float m = -INFINITY, l = 0.f;
+    for (int j = w; j <= p; j += 4) {
+        const T* krow = kc + ((size_t)table[j / page] * page + j % page) * D;
+        float kv[E], dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int c = lane + 64 * e;
+            kv[e] = c < D ? tl_to_float(krow[c]) : 0.f;
+            dot += qv[e] * kv[e];
+        }
+        dot = tl_wave_sum(dot);
+        const float m_new = fmaxf(m, dot);
+        const float corr = expf(m - m_new), pe = expf(dot - m_new);
+        l = l * corr + pe;
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[e] = acc[e] * corr + pe * kv[e];
+        m = m_new;
+    }
+    if (lane == 0) {
+        sm[w] = m;
+        sl[w] = l;
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) sacc[w][lane + 64 * e] = acc[e];
+    __syncthreads();
+    float M = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+    float f[4], L = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[i] = sm[i] > -INFINITY ? expf(sm[i] - M) : 0.f;
+        L += sl[i] * f[i];
+    }
+    T* orow = out + ((size_t)t * H + h) * D;
+    for (int c = threadIdx.x; c < D; c += 256) {
+        float v = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v += sacc[i][c] * f[i];
+        orow[c] = tl_from_float<T>(v / L);
+    }
+}
+
+extern "C" int tl_attention_wide(const void* q, const void* k_cache, int dtype, const int32_t* tables, int NB,
+                                 const int32_t* seq_of_token, const int32_t* pos, void* out, int T, int H, int D, int page,
+                                 float scale, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && H > 0 && H <= 65535 && D > 0 && D <= WIDE_MAX_D && page > 0 && NB > 0,
+                 "tl_attention_wide: bad sizes H=%d D=%d (rows of at most %d)", H, D, WIDE_MAX_D);
+    if (T == 0) return 0;
+    dim3 grid(T, H), block(256);
+    if (dtype == TL_F32)
+        hipLaunchKernelGGL(attn_wide_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_cache, tables, NB,
+                           seq_of_token, pos, (float*)out, H, D, page, scale);
+    else if (dtype == TL_BF16)
+        hipLaunchKernelGGL(attn_wide_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache, tables, NB,
+                           seq_of_token, pos, (bf16_t*)out, H, D, page, scale);
+    else return tl_fail("tl_attention_wide: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_attention_wide");
     return 0;
 }

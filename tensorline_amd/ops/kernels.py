@@ -1044,6 +1044,30 @@ def latent_prepare(proj: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor, ma
     return q_plain, q_lat
 
 
+WIDE_ROW_MAX = 1024      # the widest cached row the plain wide-row attention takes
+
+
+def wide_row_attention(q: torch.Tensor, k_cache: torch.Tensor, tables: torch.Tensor, seq_of_token: torch.Tensor,
+                       pos: torch.Tensor, heads: int, scale: float) -> torch.Tensor:
+    """Causal attention of ``heads`` query heads over one shared key/value head whose cached rows (key and
+    value at once) are wider than the matrix-core kernels take: ``q`` [T, heads * D], ``k_cache`` [pages,
+    page, 1, D] with D up to ``WIDE_ROW_MAX``.  Plain float arithmetic, a work-group per (token, head): for
+    sizes nothing else serves.  Returns [T, heads * D]."""
+    _on_gpu(q, k_cache, tables, seq_of_token, pos)
+    T = q.shape[0]
+    _check(k_cache.dim() == 4 and k_cache.is_contiguous() and k_cache.shape[2] == 1 and k_cache.dtype == q.dtype,
+           "wide_row_attention: the cache must be contiguous [pages, page, 1, D] of the queries' dtype")
+    page, D = k_cache.shape[1], k_cache.shape[3]
+    _check(D <= WIDE_ROW_MAX and q.is_contiguous() and tuple(q.shape) == (T, heads * D), "wide_row_attention: bad query layout")
+    _check(tables.dim() == 2 and tables.dtype == torch.int32 and tables.is_contiguous(), "wide_row_attention: bad page table")
+    _i32(seq_of_token, "seq_of_token", T)
+    _i32(pos, "pos", T)
+    out = torch.empty_like(q)
+    _call("tl_attention_wide", _ptr(q), _ptr(k_cache), _code(q, "wide_row_attention"), _ptr(tables), tables.shape[1],
+          _ptr(seq_of_token), _ptr(pos), _ptr(out), T, heads, D, page, ctypes.c_float(scale), _stream())
+    return out
+
+
 def head_gate(o: torch.Tensor, gate: torch.Tensor, heads: int) -> torch.Tensor:
     """``o`` [T, heads * dv], in place: head h times ``sigmoid(gate[t, h])`` (``gate`` float32, rows may be strided)."""
     _on_gpu(o, gate)

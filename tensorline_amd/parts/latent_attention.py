@@ -47,8 +47,13 @@ class LatentAttention(Part):
         # matrix-core attention kernels take (32, 64, 128, 256)
         need = self.rank + self.rot_dim
         self.cache_dim = next((d for d in kernels.MFMA_HEAD_DIMS if d >= need), 0)
-        if not self.cache_dim:
-            raise ValueError(f"{prefix}: kv_rank + rot_dim = {need} is not served: the attention kernels take rows of up to 256")
+        self.wide = not self.cache_dim
+        if self.wide:
+            # wider than those kernels take: rows in steps of 16 and the plain wide-row attention (slow;
+            # it keeps such a model served)
+            self.cache_dim = -(-need // 16) * 16
+            if self.cache_dim > kernels.WIDE_ROW_MAX:
+                raise ValueError(f"{prefix}: kv_rank + rot_dim = {need} is not served: cached rows of up to {kernels.WIDE_ROW_MAX}")
         freq, self.mag = yarn_frequencies(self.rot_dim, float(rot["base"]), rot.get("scaling"))
         self.freq = freq.to(device)
         H = self.heads
@@ -104,9 +109,12 @@ class LatentAttention(Part):
         q_plain, q_lat = kernels.latent_prepare(proj, ctx.pos, self.freq, self.mag, self.norm_w, self.eps, cache.slots,
                                                 keys, values, H, self.dim, self.rot_dim, self.rank)
         kernels.batched_linear(q_plain.view(T, H, self.dim), self.uk_t, q_lat.view(T, H, D)[:, :, :self.rank])
-        o_lat = kernels.paged_attention(q_lat, keys, values, cache.tables, ctx.seq_of_token, ctx.pos, H, 1, D, self.scale,
-                                        q_start=ctx.q_start, ctx_start=ctx.ctx_start, plan=ctx.facts,
-                                        single_seqs=ctx.extra.get("attention.single_seqs"))
+        if self.wide:
+            o_lat = kernels.wide_row_attention(q_lat, keys, cache.tables, ctx.seq_of_token, ctx.pos, H, self.scale)
+        else:
+            o_lat = kernels.paged_attention(q_lat, keys, values, cache.tables, ctx.seq_of_token, ctx.pos, H, 1, D, self.scale,
+                                            q_start=ctx.q_start, ctx_start=ctx.ctx_start, plan=ctx.facts,
+                                            single_seqs=ctx.extra.get("attention.single_seqs"))
         o = torch.empty(T, H * self.vdim, dtype=o_lat.dtype, device=o_lat.device)
         kernels.batched_linear(o_lat.view(T, H, D)[:, :, :self.rank], self.uv, o.view(T, H, self.vdim))
         gate0 = H * (self.dim + self.rot_dim) + self.rank + self.rot_dim
