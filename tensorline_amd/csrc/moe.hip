@@ -280,8 +280,8 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_kernel(const TA* __restri
 // The same product for bfloat16 operands on v_mfma_f32_16x16x32_bf16 (products exact, sums in float).
 // Tiles of BM x 128 matrix rows per work-group (GLU: 64 gate rows and the 64 up rows of the same
 // columns), k in steps of 64 through double-buffered LDS whose rows are padded to 144 bytes, so that the
-// sixteen 16-byte fragment reads of a quarter wave fall into different banks; the next step's pieces
-// wait in registers meanwhile.  Lane l = 16 g + c gives row c of a block at the eight k from 8 g on,
+// sixteen 16-byte fragment reads of a quarter wave fall into different banks; the pieces of the next two
+// steps wait in registers meanwhile (what a step costs is the chain load - registers - LDS - barrier).  Lane l = 16 g + c gives row c of a block at the eight k from 8 g on,
 // as first operand (a row of A) and as second (a row of W), and holds C[4 g + v][c] in register v.
 typedef __bf16 mg_bf16x8 __attribute__((ext_vector_type(8)));
 #define MGB_KT 64
@@ -312,14 +312,16 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
 #pragma unroll
     for (int i = 0; i < MB; ++i) acc[i][0] = acc[i][1] = (mg_f32x4){0.f, 0.f, 0.f, 0.f};
 
-    uint4 areg[A_PER], wreg[W_PER];
-    auto fetch = [&](int k0) {
+    // Two steps of look-ahead: while step s is multiplied out of LDS, the pieces of steps s + 1 and s + 2
+    // are in registers or on their way (two sets, used in turn).
+    uint4 areg[2][A_PER], wreg[2][W_PER];
+    auto fetch = [&](int k0, uint4* ar, uint4* wr) {
 #pragma unroll
         for (int it = 0; it < A_PER; ++it) {
             const int p = tid + it * MG_THREADS;
             const int r = p >> 3, k = k0 + 8 * (p & 7);
             const int src = p < A_PIECES ? arow[r] : -1;
-            areg[it] = (src >= 0 && k < K) ? *reinterpret_cast<const uint4*>(A + (size_t)src * lda + k) : make_uint4(0, 0, 0, 0);
+            ar[it] = (src >= 0 && k < K) ? *reinterpret_cast<const uint4*>(A + (size_t)src * lda + k) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int it = 0; it < W_PER; ++it) {
@@ -327,31 +329,24 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
             const int r = p >> 3, k = k0 + 8 * (p & 7);
             const int col = (GLU && r >= 64) ? n0 + r - 64 : n0 + r;
             const size_t wrow = (GLU && r >= 64) ? (size_t)N + col : (size_t)col;
-            wreg[it] = (col < N && k < K) ? *reinterpret_cast<const uint4*>(We + wrow * K + k) : make_uint4(0, 0, 0, 0);
+            wr[it] = (col < N && k < K) ? *reinterpret_cast<const uint4*>(We + wrow * K + k) : make_uint4(0, 0, 0, 0);
         }
     };
-    auto to_lds = [&](int buf) {
+    auto to_lds = [&](int buf, const uint4* ar, const uint4* wr) {
 #pragma unroll
         for (int it = 0; it < A_PER; ++it) {
             const int p = tid + it * MG_THREADS;
-            if (p < A_PIECES) *reinterpret_cast<uint4*>(&As[buf][(p >> 3) * MGB_LD + 8 * (p & 7)]) = areg[it];
+            if (p < A_PIECES) *reinterpret_cast<uint4*>(&As[buf][(p >> 3) * MGB_LD + 8 * (p & 7)]) = ar[it];
         }
 #pragma unroll
         for (int it = 0; it < W_PER; ++it) {
             const int p = tid + it * MG_THREADS;
-            *reinterpret_cast<uint4*>(&Ws[buf][(p >> 3) * MGB_LD + 8 * (p & 7)]) = wreg[it];
+            *reinterpret_cast<uint4*>(&Ws[buf][(p >> 3) * MGB_LD + 8 * (p & 7)]) = wr[it];
         }
     };
     // W rows of this wave's two blocks: GLU gate block `wave` and up block `wave`; else blocks 2 wave, 2 wave + 1
     const int wr0 = (GLU ? wave * 16 : wave * 32) + c, wr1 = (GLU ? 64 + wave * 16 : wave * 32 + 16) + c;
-
-    fetch(0);
-    to_lds(0);
-    __syncthreads();
-    int buf = 0;
-    for (int k0 = 0; k0 < K; k0 += MGB_KT) {
-        const bool more = k0 + MGB_KT < K;
-        if (more) fetch(k0 + MGB_KT);
+    auto multiply = [&](int buf) {
 #pragma unroll
         for (int s = 0; s < MGB_KT / 32; ++s) {
             const mg_bf16x8 w0 = __builtin_bit_cast(mg_bf16x8, *reinterpret_cast<const uint4*>(&Ws[buf][wr0 * MGB_LD + 32 * s + 8 * g]));
@@ -363,10 +358,27 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
                 acc[i][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, w1, acc[i][1], 0, 0, 0);
             }
         }
-        if (more) {
-            to_lds(buf ^ 1);
+    };
+
+    const int nsteps = (K + MGB_KT - 1) / MGB_KT;
+    fetch(0, areg[0], wreg[0]);
+    to_lds(0, areg[0], wreg[0]);
+    if (nsteps > 1) fetch(MGB_KT, areg[0], wreg[0]);
+    if (nsteps > 2) fetch(2 * MGB_KT, areg[1], wreg[1]);
+    __syncthreads();
+    // step s is in LDS buffer s % 2; set s % 2 holds step s + 1, the other set step s + 2
+    for (int s = 0; s < nsteps; s += 2) {
+        multiply(0);
+        if (s + 1 < nsteps) {
+            to_lds(1, areg[0], wreg[0]);
+            if (s + 3 < nsteps) fetch((s + 3) * MGB_KT, areg[0], wreg[0]);
             __syncthreads();
-            buf ^= 1;
+            multiply(1);
+            if (s + 2 < nsteps) {
+                to_lds(0, areg[1], wreg[1]);
+                if (s + 4 < nsteps) fetch((s + 4) * MGB_KT, areg[1], wreg[1]);
+                __syncthreads();
+            }
         }
     }
 
