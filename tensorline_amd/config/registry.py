@@ -76,3 +76,4 @@ def _ensure_builtin() -> None:
     # Importing the module registers it; done lazily so that config/ has no import cycle.
     import tensorline_amd.models.qwen2  # noqa: F401
     import tensorline_amd.models.samovik  # noqa: F401
+    import tensorline_amd.models.tumitar  # noqa: F401

@@ -9,12 +9,13 @@ void tl_attention_generic_bf16(const AgLaunch& a);
 // the keys into runs of split_keys (a multiple of 64) at absolute positions, one work-group each,
 // and a second kernel merges them: for steps of few tokens with long contexts, which would
 // otherwise be walked by one work-group per sequence and key/value head.  nsplit * split_keys must
-// cover the longest context; ws holds T * nq * nsplit * (d + 2) floats.
+// cover the longest context; ws holds T * nq * nsplit * (d + 2) floats.  sink != 0: one is added to the
+// softmax's denominator (a key of score 0 that has no value).
 extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                     const int32_t* tables, int NB, const int32_t* q_start, const int32_t* pos,
                                     void* out, int out_stride, int dtype, int T, int S, int max_query_len, int nq, int nkv,
                                     int d, int bs, int window, float scale, int nsplit, int split_keys, float* ws,
-                                    hipStream_t stream) {
+                                    int sink, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && d > 0 && bs > 0 && NB > 0,
                  "tl_attention_generic: bad sizes T=%d S=%d nq=%d nkv=%d d=%d page=%d NB=%d", T, S, nq, nkv, d, bs, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_generic: %d query heads are not a multiple of %d key/value heads", nq, nkv);
@@ -52,7 +53,7 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
     a.tiles_per_seq = tiles_per_seq; a.QT = QT; a.GC = GC; a.nq = nq; a.nkv = nkv; a.d = d; a.bs = bs; a.bs_shift = bs_shift;
     a.window = window; a.nsplit = nsplit; a.split_keys = split_keys; a.scale = scale; a.keys_over_waves = keys_over_waves;
     a.grid = dim3((unsigned)groups, nkv, chunks * nsplit);
-    a.smem = smem; a.stream = stream;
+    a.smem = smem; a.stream = stream; a.sink = sink;
     if (dtype == TL_F32)
         ag_launch_all<float>(a);
     else if (dtype == TL_BF16)

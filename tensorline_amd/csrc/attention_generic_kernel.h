@@ -98,7 +98,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
     T* __restrict__ out, int out_stride, int tiles_per_seq, int QT, int GC, int nq, int nkv, int bs, int bs_shift,
-    int window, float scale, int nsplit, int split_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
+    int window, float scale, int nsplit, int split_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml, int sink) {
     constexpr int d = DB * 16;
     constexpr int KT = AG_KT(d, KW);
     extern __shared__ float smem[];
@@ -421,7 +421,8 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
         if (my_pos[v] < 0) continue;
         const int row = wave * AG_WROWS + 4 * lg + v;
         const int i = row / GC, g = row - i * GC;
-        const float inv = (l[v] > 0.f) ? 1.f / l[v] : 0.f;
+        // with a sink one is added to the denominator: a key of score 0 that has no value
+        const float inv = (l[v] > 0.f) ? 1.f / (sink ? l[v] + expf(-m[v]) : l[v]) : 0.f;
         T* orow = out + (size_t)(t_first + i) * out_stride + (size_t)(kvh * G + g0 + g) * d;
 #pragma unroll
         for (int db = 0; db < DB; ++db) orow[db * 16 + li] = tl_from_float<T>(acc[db][v] * inv);
@@ -445,7 +446,7 @@ __device__ __forceinline__ float ag_group_max(float v, float* red) {   // red: o
 template <typename T>
 __global__ __launch_bounds__(256) void attn_generic_merge_kernel(const float* __restrict__ ws_o,
                                                                  const float* __restrict__ ws_ml, T* __restrict__ out,
-                                                                 int out_stride, int nq, int d, int nsplit) {
+                                                                 int out_stride, int nq, int d, int nsplit, int sink) {
     __shared__ float wgt[AG_MAX_SPLITS], wl[AG_MAX_SPLITS], red[4];
     const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const size_t base = ((size_t)t * nq + h) * nsplit;
@@ -472,6 +473,7 @@ __global__ __launch_bounds__(256) void attn_generic_merge_kernel(const float* __
     if (tid >= d) return;
     float den = 0.f;
     for (int sp = 0; sp < nsplit; ++sp) den += wl[sp];
+    if (sink && den > 0.f) den += expf(-M);              // the sink: a key of score 0 without a value
     const float* acc = ws_o + base * d + tid;
     float num = 0.f;
     for (int s0 = 0; s0 < nsplit; s0 += 8) {
@@ -495,7 +497,7 @@ struct AgLaunch {
     const int32_t *tables, *q_start, *pos;
     void* out;
     float *ws_o, *ws_ml;
-    int q_stride, NB, out_stride, T, tiles_per_seq, QT, GC, nq, nkv, d, bs, bs_shift, window, nsplit, split_keys;
+    int q_stride, NB, out_stride, T, tiles_per_seq, QT, GC, nq, nkv, d, bs, bs_shift, window, nsplit, split_keys, sink;
     float scale;
     bool keys_over_waves;
     dim3 grid;
@@ -514,7 +516,7 @@ static void ag_launch_all(const AgLaunch& a) {
     hipLaunchKernelGGL((attn_generic_kernel<TT, DB, KWV>), a.grid, block, a.smem, a.stream, (const TT*)a.q,           \
                        a.q_stride, (const TT*)a.k_cache, (const TT*)a.v_cache, a.tables, a.NB, a.q_start, a.pos,      \
                        (TT*)a.out, a.out_stride, a.tiles_per_seq, a.QT, a.GC, a.nq, a.nkv, a.bs, a.bs_shift, a.window, \
-                       a.scale, a.nsplit, a.split_keys, a.ws_o, a.ws_ml)
+                       a.scale, a.nsplit, a.split_keys, a.ws_o, a.ws_ml, a.sink)
 #define AG_CASE(DB)                                                                                                   \
     case DB:                                                                                                          \
         if (a.keys_over_waves) AG_LAUNCH_KW(DB, true); else AG_LAUNCH_KW(DB, false);                                  \
@@ -527,5 +529,5 @@ static void ag_launch_all(const AgLaunch& a) {
 #undef AG_LAUNCH_KW
     if (a.nsplit > 1)
         hipLaunchKernelGGL(attn_generic_merge_kernel<TT>, dim3(a.T, a.nq), dim3(256), 0, a.stream, a.ws_o, a.ws_ml,
-                           (TT*)a.out, a.out_stride, a.nq, a.d, a.nsplit);
+                           (TT*)a.out, a.out_stride, a.nq, a.d, a.nsplit, a.sink);
 }

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int nq, int nkv, int bs, int bs_shift, int window, float scale, int nsplit,
-    int split_blocks, const int32_t* __restrict__ seq_list, int skip_single) {
+    int split_blocks, const int32_t* __restrict__ seq_list, int skip_single, int sink) {
     constexpr int D = DC * 32;
     constexpr int DB = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -279,6 +279,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
         l_tot += __shfl_xor(l_tot, 16, TL_WAVE);
         l_tot += __shfl_xor(l_tot, 32, TL_WAVE);
         if (nsplit == 1) {
+            if (sink) l_tot += exp2f(-m_run[j]);             // the sink: a key of score 0 without a value
             const float inv = 1.0f / l_tot;
             bf16_t* op = out + (size_t)row_col[j] * out_stride + (size_t)head_col[j] * D + 4 * g;
 #pragma unroll
@@ -553,7 +554,7 @@ __global__ __launch_bounds__(CH * WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int S, int nq, int nkv, int bs,
-    int bs_shift, int window, float scale, int skip_single) {
+    int bs_shift, int window, float scale, int skip_single, int sink) {
     constexpr int THREADS = CH * WAVES * 64;
     constexpr int WCOLS = NT * 16;                       // columns of a wave; WAVES * WCOLS = 128 per work-group
     constexpr int D = DC * 32;
@@ -798,6 +799,7 @@ __global__ __launch_bounds__(CH * WAVES * 64, 32 / WAVES) void attn_tile_kernel(
             for (int db = 0; db < DB; ++db)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) acc[j][db][i] = acc[j][db][i] * w0 + hand[(j * PER + 2 + db * 4 + i) * 64] * w1;
+            m_run[j] = mm;                                   // what the sums now refer to
         }
     }
 
@@ -807,6 +809,7 @@ __global__ __launch_bounds__(CH * WAVES * 64, 32 / WAVES) void attn_tile_kernel(
         float l_tot = l_run[j];
         l_tot += __shfl_xor(l_tot, 16, TL_WAVE);
         l_tot += __shfl_xor(l_tot, 32, TL_WAVE);
+        if (sink) l_tot += exp2f(-m_run[j]);                 // the sink: a key of score 0 without a value
         const float inv = 1.0f / l_tot;
         bf16_t* op = out + (size_t)row_col[j] * out_stride + (size_t)head_col[j] * D + 4 * g;
 #pragma unroll
@@ -839,7 +842,7 @@ template <int AM_MERGE_THREADS>
 __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml, const int32_t* __restrict__ pos,
     bf16_t* __restrict__ out, int out_stride, int nq, int D, int nsplit, int split_blocks, int window,
-    const int32_t* __restrict__ seq_list, const int32_t* __restrict__ q_start) {
+    const int32_t* __restrict__ seq_list, const int32_t* __restrict__ q_start, int sink) {
     __shared__ float wgt[AM_MAX_SPLITS];
     __shared__ float red_m[AM_MERGE_THREADS / 64], red_l[AM_MERGE_THREADS / 64];
     __shared__ float4 part[AM_MERGE_THREADS];
@@ -893,6 +896,7 @@ __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     float L = red_l[0];
 #pragma unroll
     for (int w = 1; w < AM_MERGE_THREADS / 64; ++w) L += red_l[w];
+    if (sink) L += exp2f(-M);                                // the sink: a key of score 0 without a value
     float4 o4 = zero4;
 #pragma unroll
     for (int k = 0; k < AM_MERGE_AHEAD; ++k) {
@@ -929,18 +933,18 @@ static void launch_attn(int NT, dim3 grid, int wg_waves, hipStream_t stream, con
                         const bf16_t* vc, const int32_t* tables, int NB, const int32_t* q_start,
                         const int32_t* ctx_start, bf16_t* out, int out_stride, float* ws_o, float* ws_ml, int nq, int nkv,
                         int bs, int window, float scale, int nsplit, int split_blocks, const int32_t* seq_list,
-                        int skip_single) {
+                        int skip_single, int sink) {
     int bs_shift = -1;                               // pages of a power of two of tokens: a shift finds the page
     if ((bs & (bs - 1)) == 0)
         for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
     if (NT == 1)
         hipLaunchKernelGGL((attn_mfma_kernel<DC, 1>), grid, dim3(64 * wg_waves), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
                            ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
-                           split_blocks, seq_list, skip_single);
+                           split_blocks, seq_list, skip_single, sink);
     else
         hipLaunchKernelGGL((attn_mfma_kernel<DC, 2>), grid, dim3(64 * wg_waves), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
                            ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
-                           split_blocks, seq_list, skip_single);
+                           split_blocks, seq_list, skip_single, sink);
 }
 
 // q: bfloat16 [T, >= nq*d] (row stride q_stride); k_cache [pages, page, nkv, d]; v_cache
@@ -957,12 +961,13 @@ static void launch_attn(int NT, dim3 grid, int wg_waves, hipStream_t stream, con
 // computed, with split keys, and the workspace then holds n_list rows instead of T), and one
 // with skip_single != 0, which leaves sequences of one token out.
 // total_groups128: the sum over the sequences of ceil(n_s * G / 128), that kernel's grid.
+// sink != 0: one is added to the softmax's denominator (a key of score 0 that has no value).
 extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
                                  const int32_t* pos, void* out, int out_stride, float* ws_o, float* ws_ml, int T, int S,
                                  int nq, int nkv, int d, int bs, int window, float scale, int NT, int max_tile_groups,
                                  int nsplit, int split_blocks, int shared, int total_groups128,
-                                 const int32_t* seq_list, int n_list, int skip_single, hipStream_t stream) {
+                                 const int32_t* seq_list, int n_list, int skip_single, int sink, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_mfma: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_mfma: %d query heads are not a multiple of %d key/value heads", nq, nkv);
     TL_CHECK_ARG(d == 32 || d == 64 || d == 128 || d == 256, "tl_attention_mfma: head size %d is not one of 32, 64, 128, 256", d);
@@ -1009,11 +1014,11 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
         if (chains == 2)                                                                                              \
             hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT, 2>), sgrid, dim3(2 * 64 * 8 / AT_NT), lds,    \
                                stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, \
-                               S, nq, nkv, bs, bs_shift, window, scale, skip_single);                                 \
+                               S, nq, nkv, bs, bs_shift, window, scale, skip_single, sink);                                 \
         else                                                                                                          \
             hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT, 1>), sgrid, dim3(64 * 8 / AT_NT), lds,        \
                                stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, \
-                               S, nq, nkv, bs, bs_shift, window, scale, skip_single);                                 \
+                               S, nq, nkv, bs, bs_shift, window, scale, skip_single, sink);                                 \
     } while (0)
         if (d == 32) TL_TILE_CASE(1);
         else if (d == 64) TL_TILE_CASE(2);
@@ -1024,25 +1029,25 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     }
     if (d == 32)
         launch_attn<1>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single, sink);
     else if (d == 64)
         launch_attn<2>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single, sink);
     else if (d == 128)
         launch_attn<4>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single, sink);
     else
         launch_attn<8>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single, sink);
     TL_CHECK_LAUNCH("tl_attention_mfma");
     if (nsplit > 1) {
         const int merge_rows = seq_list ? n_list : T;
         if (nsplit > 32)
             hipLaunchKernelGGL(attn_merge_kernel<256>, dim3(merge_rows, nq), dim3(256), 0, stream, ws_o, ws_ml, pos,
-                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window, seq_list, q_start);
+                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window, seq_list, q_start, sink);
         else
             hipLaunchKernelGGL(attn_merge_kernel<128>, dim3(merge_rows, nq), dim3(128), 0, stream, ws_o, ws_ml, pos,
-                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window, seq_list, q_start);
+                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window, seq_list, q_start, sink);
         TL_CHECK_LAUNCH("tl_attention_mfma merge");
     }
     return 0;

@@ -220,7 +220,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int S, int nq, int nkv, int bs,
-    int bs_shift, int window, float scale, int skip_single) {
+    int bs_shift, int window, float scale, int skip_single, int sink) {
     constexpr int THREADS = WAVES * 64;
     constexpr int WGC = WAVES * 32;           // columns of a work-group
     constexpr int D = DC * 32, KS = D / 16, DT = D / 32;
@@ -421,7 +421,8 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
 #undef T32_LANDED
 
     if (!valid) return;
-    const float inv = 1.0f / t32_halves_sum(l_run);
+    // with a sink one is added to the denominator: a key of score 0 that has no value
+    const float inv = 1.0f / (t32_halves_sum(l_run) + (sink ? exp2f(-m_run) : 0.f));
     // register r of row tile m is dim 32 m + 8 (r / 4) + 4 h + r % 4: four consecutive dims per store
     bf16_t* op = out + (size_t)row_out * out_stride + (size_t)head * D + 4 * h;
 #pragma unroll
@@ -455,7 +456,7 @@ extern "C" int tl_attention_tile32_columns(int waves) { return 32 * waves; }
 extern "C" int tl_attention_tile32(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                    const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
                                    void* out, int out_stride, int T, int S, int nq, int nkv, int d, int bs, int window,
-                                   float scale, int waves, int total_groups, int skip_single, hipStream_t stream) {
+                                   float scale, int waves, int total_groups, int skip_single, int sink, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_tile32: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_tile32: %d query heads are not a multiple of %d key/value heads", nq, nkv);
     TL_CHECK_ARG(tl_attention_tile32_takes(d, bs, NB, S, waves),
@@ -476,7 +477,7 @@ extern "C" int tl_attention_tile32(const void* q, int q_stride, const void* k_ca
     const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
 #define T32_LAUNCH(DCV, WV)                                                                                             \
     hipLaunchKernelGGL((attn_tile32_kernel<DCV, WV>), grid, dim3(64 * WV), lds, stream, qq, q_stride, kk, vv, tables, NB, \
-                       q_start, ctx_start, (bf16_t*)out, out_stride, S, nq, nkv, bs, bs_shift, window, scale, skip_single)
+                       q_start, ctx_start, (bf16_t*)out, out_stride, S, nq, nkv, bs, bs_shift, window, scale, skip_single, sink)
     if (d == 64 && waves == 4) T32_LAUNCH(2, 4);
     else if (d == 64) T32_LAUNCH(2, 8);
     else if (waves == 4) T32_LAUNCH(4, 4);

@@ -25,11 +25,11 @@ extern "C" const char* tl_last_error() { return g_tl_error; }
 extern "C" int tl_abi_version() { return 1; }
 
 // ---- embedding gather ----------------------------------------------------------------------
-// x[t, :] = float(table[ids[t], :]).  An id outside [0, V) gives a row of NaN instead of a fault;
+// x[t, :] = float(table[ids[t], :]) * scale.  An id outside [0, V) gives a row of NaN instead of a fault;
 // callers validate ids on the host.
 template <typename T>
 __global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
-                             float* __restrict__ x, int H, int V) {
+                             float* __restrict__ x, int H, int V, float scale) {
     const int t = blockIdx.x;
     const int id = ids[t];
     float* xr = x + (size_t)t * H;
@@ -38,18 +38,18 @@ __global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restric
         return;
     }
     const T* row = table + (size_t)id * H;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) xr[c] = tl_to_float(row[c]);
+    for (int c = threadIdx.x; c < H; c += blockDim.x) xr[c] = tl_to_float(row[c]) * scale;
 }
 
 extern "C" int tl_embed(const int32_t* ids, const void* table, int table_dtype, float* x, int T, int H, int V,
-                        hipStream_t stream) {
+                        float scale, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && H > 0 && V > 0, "tl_embed: bad sizes T=%d H=%d V=%d", T, H, V);
     if (T == 0) return 0;
     dim3 grid(T), block(256);
     if (table_dtype == TL_F32)
-        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, (const float*)table, x, H, V);
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, (const float*)table, x, H, V, scale);
     else if (table_dtype == TL_BF16)
-        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, x, H, V);
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, x, H, V, scale);
     else
         return tl_fail("tl_embed: unknown dtype %d", table_dtype);
     TL_CHECK_LAUNCH("tl_embed");

@@ -1,12 +1,14 @@
 // Routed experts: choice of experts per token, the tokens of each expert gathered into row tiles,
 // the experts' products as one grouped launch each, and the weighted sum per token.
 //
-//   tl_moe_route    per token: the `top` largest router logits (lowest index wins a tie) and the
-//                   softmax over those alone                      -> expert ids, weights [T, top]
+//   tl_moe_route    per token: the `top` largest router logits (lowest index wins a tie) and their weights:
+//                   the softmax over those alone, or scale * sigmoid of each  -> expert ids, weights [T, top]
 //   tl_moe_sort     the (token, choice) pairs ordered by expert and cut into row tiles of BM rows that
 //                   hold one expert's pairs only                 -> order, tiles
-//   tl_moe_gemm     a product per tile with its expert's matrix: gate/up with the clamped gated
-//                   activation in the epilogue, or down, which scatters rows back to their pairs
+//   tl_moe_gemm     a product per tile with its expert's matrix: gate/up with the gated activation
+//                   min(g, limit) sigmoid(alpha min(g, limit)) (clamp(u, +-limit) + shift) in the epilogue
+//                   (limit = infinity, alpha = 1, shift = 0: silu(g) u), or down, which scatters rows back
+//                   to their pairs
 //   tl_moe_combine  out[t] = sum over the token's choices, in the order of its choices, of weight *
 //                   row (+ a shared expert's output)
 //
@@ -26,7 +28,8 @@
 // A wave per token: lane l looks at logits l, l + 64, ...; the largest not yet chosen is found by a
 // butterfly over (value, index), equal values going to the lower index; lane c keeps the c-th choice.
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ldl, int32_t* __restrict__ ids,
-                                                        float* __restrict__ weights, int T, int E, int top) {
+                                                        float* __restrict__ weights, int T, int E, int top, int mode,
+                                                        float scale) {
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (t >= T) return;
@@ -61,6 +64,13 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
             my_id = be;
         }
     }
+    if (mode == 1) {                    // every chosen expert by its own score: scale * sigmoid(logit)
+        if (lane < top) {
+            ids[(size_t)t * top + lane] = my_id;
+            weights[(size_t)t * top + lane] = scale * (1.0f / (1.0f + expf(-my_val)));
+        }
+        return;
+    }
     const float largest = __shfl(my_val, 0, 64);
     const float ex = lane < top ? expf(my_val - largest) : 0.f;
     const float sum = tl_wave_sum(ex);
@@ -70,12 +80,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
 }
 
-extern "C" int tl_moe_route(const float* logits, int ldl, int32_t* ids, float* weights, int T, int E, int top,
-                            hipStream_t stream) {
+// mode 0: weights = softmax over the chosen logits; mode 1: weights = scale * sigmoid(chosen logit).
+extern "C" int tl_moe_route(const float* logits, int ldl, int32_t* ids, float* weights, int T, int E, int top, int mode,
+                            float scale, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && E > 0 && top > 0 && top <= E && top <= MOE_MAX_TOP && E <= MOE_MAX_EXPERTS && ldl >= E,
                  "tl_moe_route: bad sizes E=%d top=%d", E, top);
+    TL_CHECK_ARG(mode == 0 || mode == 1, "tl_moe_route: unknown weighting %d", mode);
     if (T == 0) return 0;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(tl_ceil_div(T, 4)), dim3(256), 0, stream, logits, ldl, ids, weights, T, E, top);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(tl_ceil_div(T, 4)), dim3(256), 0, stream, logits, ldl, ids, weights, T, E, top, mode, scale);
     TL_CHECK_LAUNCH("tl_moe_route");
     return 0;
 }
@@ -170,7 +182,7 @@ template <typename TA, typename TW, typename TO, int MB, int NB, bool GLU>
 __global__ __launch_bounds__(MG_THREADS) void moe_gemm_kernel(const TA* __restrict__ A, int lda, const TW* __restrict__ W,
                                                              TO* __restrict__ C, int ldc, const int32_t* __restrict__ order,
                                                              const int32_t* __restrict__ tiles, int top, int N, int K,
-                                                             int a_vec, int w_vec, float limit, float alpha) {
+                                                             int a_vec, int w_vec, float limit, float alpha, float shift) {
     constexpr int BM = MB * 16, BN = 4 * NB * 16, WR = GLU ? 2 * BN : BN, NW = GLU ? 2 * NB : NB;
     constexpr int A_PIECES = BM * 4, W_PIECES = WR * 4;
     constexpr int A_PER = (A_PIECES + MG_THREADS - 1) / MG_THREADS, W_PER = (W_PIECES + MG_THREADS - 1) / MG_THREADS;
@@ -269,7 +281,7 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_kernel(const TA* __restri
                 if (GLU) {
                     const float g = fminf(acc[i][j][v], limit);
                     const float u = fminf(fmaxf(acc[i][NB + j][v], -limit), limit);
-                    C[(size_t)(place0 + r) * ldc + n] = tl_from_float<TO>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
+                    C[(size_t)(place0 + r) * ldc + n] = tl_from_float<TO>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + shift));
                 } else {
                     C[(size_t)order[place0 + r] * ldc + n] = tl_from_float<TO>(acc[i][j][v]);
                 }
@@ -292,7 +304,7 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
                                                                   const bf16_t* __restrict__ W, void* __restrict__ Cv, int ldc,
                                                                   const int32_t* __restrict__ order,
                                                                   const int32_t* __restrict__ tiles, int top, int N, int K,
-                                                                  float limit, float alpha) {
+                                                                  float limit, float alpha, float shift) {
     constexpr int BM = MB * 16, WR = 128, BN = GLU ? 64 : 128;
     constexpr int A_PIECES = BM * 8, W_PIECES = WR * 8;
     constexpr int A_PER = (A_PIECES + MG_THREADS - 1) / MG_THREADS, W_PER = W_PIECES / MG_THREADS;
@@ -394,7 +406,7 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
                 const float gt = fminf(acc[i][0][v], limit);
                 const float up = fminf(fmaxf(acc[i][1][v], -limit), limit);
                 reinterpret_cast<bf16_t*>(Cv)[(size_t)(place0 + r) * ldc + n] =
-                    tl_from_float<bf16_t>(gt * (1.0f / (1.0f + expf(-alpha * gt))) * (up + 1.0f));
+                    tl_from_float<bf16_t>(gt * (1.0f / (1.0f + expf(-alpha * gt))) * (up + shift));
             } else {
                 float* crow = reinterpret_cast<float*>(Cv) + (size_t)order[place0 + r] * ldc;
 #pragma unroll
@@ -411,7 +423,7 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
 // tl_moe_sort can have made: P / BM + E.
 extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, int w_dtype, void* C, int c_dtype, int ldc,
                            const int32_t* order, const int32_t* tiles, int max_tiles, int BM, int top, int N, int K, int glu,
-                           float limit, float alpha, hipStream_t stream) {
+                           float limit, float alpha, float shift, hipStream_t stream) {
     TL_CHECK_ARG(N > 0 && K > 0 && lda >= K && ldc >= N && top > 0 && (BM == 16 || BM == 64), "tl_moe_gemm: bad sizes N=%d K=%d BM=%d", N, K, BM);
     TL_CHECK_ARG(max_tiles >= 0 && max_tiles <= 65535, "tl_moe_gemm: %d row tiles are too many for one launch", max_tiles);
     if (max_tiles == 0) return 0;
@@ -421,7 +433,7 @@ extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, i
 #define GO(TA, TW, TO, MB, NB, GLU)                                                                                       \
     hipLaunchKernelGGL((moe_gemm_kernel<TA, TW, TO, MB, NB, GLU>), dim3(tl_ceil_div(N, 4 * NB * 16), max_tiles),          \
                        dim3(MG_THREADS), 0, stream, (const TA*)A, lda, (const TW*)W, (TO*)C, ldc, order, tiles, top, N, K, \
-                       a_vec, w_vec, limit, alpha)
+                       a_vec, w_vec, limit, alpha, shift)
 #define GO_BM(TA, TW, TO, GLU)                 \
     do {                                       \
         if (BM == 16) GO(TA, TW, TO, 1, 1, GLU); \
@@ -431,7 +443,7 @@ extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, i
     if (bf && K % 8 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0) {
 #define GO_BF(MB, GLU)                                                                                                   \
     hipLaunchKernelGGL((moe_gemm_bf16_kernel<MB, GLU>), dim3(tl_ceil_div(N, GLU ? 64 : 128), max_tiles), dim3(MG_THREADS), 0, \
-                       stream, (const bf16_t*)A, lda, (const bf16_t*)W, C, ldc, order, tiles, top, N, K, limit, alpha)
+                       stream, (const bf16_t*)A, lda, (const bf16_t*)W, C, ldc, order, tiles, top, N, K, limit, alpha, shift)
         if (glu) {
             if (BM == 16) GO_BF(1, true);
             else GO_BF(4, true);

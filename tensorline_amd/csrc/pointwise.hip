@@ -77,16 +77,24 @@ extern "C" int tl_add_cast(float* x, const float* res, void* out, int out_dtype,
 }
 
 // ---- element-wise functions ------------------------------------------------------------------------
-// kind 0: tanh.  float in, float or bfloat16 out.
+// kind 0: tanh; kind 1: the square of relu.  float in, float or bfloat16 out.
 template <typename O>
 __global__ void unary_kernel(const float* __restrict__ in, O* __restrict__ out, size_t n, int kind) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    out[i] = tl_from_float<O>(tanhf(in[i]));
+    const float z = in[i];
+    float r;
+    if (kind == 0) {
+        r = tanhf(z);
+    } else {
+        const float p = fmaxf(z, 0.f);
+        r = p * p;
+    }
+    out[i] = tl_from_float<O>(r);
 }
 
 extern "C" int tl_unary(const float* in, void* out, int out_dtype, long long n, int kind, hipStream_t stream) {
-    TL_CHECK_ARG(n >= 0 && kind == 0, "tl_unary: bad arguments");
+    TL_CHECK_ARG(n >= 0 && (kind == 0 || kind == 1), "tl_unary: bad arguments");
     if (n == 0) return 0;
     dim3 grid((unsigned)((n + 255) / 256)), block(256);
     if (out_dtype == TL_F32) hipLaunchKernelGGL(unary_kernel<float>, grid, block, 0, stream, in, (float*)out, (size_t)n, kind);
@@ -131,7 +139,8 @@ extern "C" int tl_clamp_glu(const void* gu, int in_dtype, void* out, int out_dty
 // ---- gated normalisation over groups of columns ----------------------------------------------------
 // o float [T, N] in groups of `group` columns (a head, or the whole row): every group is divided by
 // its root mean square (eps inside the root), times weight[c], times the gate: sigmoid(gate) for
-// gate_act 0, silu(gate) for 1.  gate float [T, ldg].  One wave per group.
+// gate_act 0, silu(gate) for 1.  gate_act 2 puts the gate first: o * silu(gate) is what is divided by
+// its root mean square, then times weight[c].  gate float [T, ldg].  One wave per group.
 template <typename O>
 __global__ void gated_group_norm_kernel(const float* __restrict__ o, int ldo, const float* __restrict__ weight,
                                         const float* __restrict__ gate, int ldg, O* __restrict__ out, int N, int group,
@@ -141,15 +150,27 @@ __global__ void gated_group_norm_kernel(const float* __restrict__ o, int ldo, co
     const int groups = N / group;
     for (int g = wave; g < groups; g += nwaves) {
         const float* row = o + (size_t)t * ldo + g * group;
+        const float* grow = gate + (size_t)t * ldg + g * group;
         float ss = 0.f;
-        for (int c = lane; c < group; c += 64) ss += row[c] * row[c];
+        if (gate_act == 2) {
+            for (int c = lane; c < group; c += 64) {
+                const float v = row[c] * pw_silu(grow[c]);
+                ss += v * v;
+            }
+        } else {
+            for (int c = lane; c < group; c += 64) ss += row[c] * row[c];
+        }
         ss = tl_wave_sum(ss);
         const float rstd = 1.0f / sqrtf(ss / (float)group + eps);
         for (int c = lane; c < group; c += 64) {
             const int n = g * group + c;
-            const float z = gate[(size_t)t * ldg + n];
-            const float gv = gate_act == 0 ? pw_sigmoid(z) : pw_silu(z);
-            out[(size_t)t * N + n] = tl_from_float<O>(row[c] * rstd * weight[n] * gv);
+            const float z = grow[c];
+            if (gate_act == 2) {
+                out[(size_t)t * N + n] = tl_from_float<O>(row[c] * pw_silu(z) * rstd * weight[n]);
+            } else {
+                const float gv = gate_act == 0 ? pw_sigmoid(z) : pw_silu(z);
+                out[(size_t)t * N + n] = tl_from_float<O>(row[c] * rstd * weight[n] * gv);
+            }
         }
     }
 }
@@ -441,5 +462,98 @@ extern "C" int tl_attention_wide(const void* q, const void* k_cache, int dtype, 
                            seq_of_token, pos, (bf16_t*)out, H, D, page, scale);
     else return tl_fail("tl_attention_wide: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("tl_attention_wide");
+    return 0;
+}
+
+// ---- queries and keys normed over the whole projection, a query factor by position, the cache write ----
+// proj float [T, ldp] = [q: H*d | k: G*d | v: G*dv] (biases added already).  Per token:
+//   * q and k are each divided by the root mean square of their whole row (all heads at once, eps inside
+//     the root) and multiplied by a weight per column (wq [H*d], wk [G*d]; null: no norm);
+//   * q is multiplied by 1 + coef * ln(floor((pos + 1) / every) + 1) (every <= 0: no factor);
+//   * q goes to q_out [T, H*D], every head padded with zeros from d to D;
+//   * k goes into the cache at `slot` ([pages, page, G, D], zeros from d to D), v with a page's tokens
+//     innermost ([pages, G, D, page], zeros from dv to D).
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_store_kernel(
+    const float* __restrict__ proj, int ldp, const int32_t* __restrict__ pos, const float* __restrict__ wq,
+    const float* __restrict__ wk, float eps, float coef, int every, const int32_t* __restrict__ slots,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int d, int dv, int D, int page) {
+    __shared__ float red[16];
+    const int t = blockIdx.x;
+    const float* q = proj + (size_t)t * ldp;
+    const float* k = q + H * d;
+    const float* v = k + G * d;
+    float rq = 1.f, rk = 1.f;
+    if (wq) {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < H * d; c += blockDim.x) ss += q[c] * q[c];
+        ss = tl_block_sum(ss, red);
+        rq = 1.0f / sqrtf(ss / (float)(H * d) + eps);
+    }
+    if (wk) {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < G * d; c += blockDim.x) ss += k[c] * k[c];
+        ss = tl_block_sum(ss, red);
+        rk = 1.0f / sqrtf(ss / (float)(G * d) + eps);
+    }
+    float temp = 1.f;
+    if (every > 0) temp = 1.0f + coef * logf((float)((pos[t] + 1) / every) + 1.0f);
+    for (int idx = threadIdx.x; idx < H * D; idx += blockDim.x) {
+        const int h = idx / D, c = idx - h * D;
+        float o = 0.f;
+        if (c < d) {
+            const int n = h * d + c;
+            o = wq ? q[n] * rq * wq[n] * temp : q[n] * temp;
+        }
+        q_out[(size_t)t * H * D + idx] = tl_from_float<T>(o);
+    }
+    const int slot = slots[t];
+    if (slot < 0) return;
+    const size_t pg = (size_t)slot / page, within = (size_t)slot % page;
+    for (int idx = threadIdx.x; idx < G * D; idx += blockDim.x) {
+        const int h = idx / D, c = idx - h * D;
+        float kv = 0.f, vv = 0.f;
+        if (c < d) {
+            const int n = h * d + c;
+            kv = wk ? k[n] * rk * wk[n] : k[n];
+        }
+        if (c < dv) vv = v[h * dv + c];
+        k_cache[(size_t)slot * G * D + idx] = tl_from_float<T>(kv);
+        v_cache[(pg * G * D + idx) * page + within] = tl_from_float<T>(vv);
+    }
+}
+
+extern "C" int tl_qk_norm_store(const float* proj, int ldp, const int32_t* pos, const float* wq, const float* wk, float eps,
+                                float coef, int every, const int32_t* slots, void* q_out, void* k_cache, void* v_cache,
+                                int dtype, int T, int H, int G, int d, int dv, int D, int page, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && H > 0 && G > 0 && d > 0 && dv > 0 && D >= d && D >= dv && page > 0,
+                 "tl_qk_norm_store: bad sizes H=%d G=%d d=%d dv=%d D=%d", H, G, d, dv, D);
+    TL_CHECK_ARG(ldp >= H * d + G * d + G * dv, "tl_qk_norm_store: the projection's rows are too short");
+    TL_CHECK_ARG((wq == nullptr) == (wk == nullptr), "tl_qk_norm_store: queries and keys are normed together or not at all");
+    if (T == 0) return 0;
+    dim3 grid(T), block(256);
+    if (dtype == TL_F32)
+        hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, 0, stream, proj, ldp, pos, wq, wk, eps, coef, every, slots,
+                           (float*)q_out, (float*)k_cache, (float*)v_cache, H, G, d, dv, D, page);
+    else if (dtype == TL_BF16)
+        hipLaunchKernelGGL(qk_norm_store_kernel<bf16_t>, grid, block, 0, stream, proj, ldp, pos, wq, wk, eps, coef, every, slots,
+                           (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, H, G, d, dv, D, page);
+    else return tl_fail("tl_qk_norm_store: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_qk_norm_store");
+    return 0;
+}
+
+// ---- a weighted sum of two float tensors -------------------------------------------------------------------
+// out = a * x + b * y, element by element (out may be x or y).
+__global__ void scaled_sum_kernel(const float* x, const float* y, float* out, float a, float b, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a * x[i] + b * y[i];
+}
+
+extern "C" int tl_scaled_sum(const float* x, const float* y, float* out, float a, float b, long long n, hipStream_t stream) {
+    TL_CHECK_ARG(n >= 0, "tl_scaled_sum: bad size");
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(scaled_sum_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, y, out, a, b, (size_t)n);
+    TL_CHECK_LAUNCH("tl_scaled_sum");
     return 0;
 }

@@ -37,7 +37,7 @@ class TraceError(RuntimeError):
 class TraceSession:
     """Live requests of a trace and the cache they share."""
 
-    def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 8, graphs: bool = False):
+    def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 4, graphs: bool = False):
         """``max_tokens``: the most tokens live requests hold at any time (each request's count
         rounded up to 64); ``max_requests``: the most requests live at a time.  ``graphs``: steps
         that are pure decoding replay a HIP graph, as the engine's do, instead of running eagerly."""
@@ -107,7 +107,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64); sizes the cache")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
-    ap.add_argument("--max-requests", type=int, default=8, help="most requests live at any time")
+    ap.add_argument("--max-requests", type=int, default=4, help="most requests live at any time (state slots)")
     ap.add_argument("--graphs", action="store_true", help="replay HIP graphs for steps that only decode, as serving does")
     ap.add_argument("--device", default="cuda:0")
     return ap

@@ -130,6 +130,9 @@ class DecoderModel:
         takes no ``after=`` (then it returns a tensor, which everybody takes)."""
         takers = [self.blocks[e.layer] for e in self.schedule]
         intakes = [b.intake() if hasattr(b, "intake") else Intake() for b in takers[1:]] + [self._tail_intake()]
+        # an entry that adds the embedding output takes what runs before it as a plain tensor
+        intakes = [Intake() if n + 1 < len(self.schedule) and self.schedule[n + 1].add_input else it
+                   for n, it in enumerate(intakes)]
         return [nxt if hasattr(b, "intake") else None for b, nxt in zip(takers, intakes)]
 
     def step_vectors(self, facts) -> dict:
@@ -140,7 +143,8 @@ class DecoderModel:
             seen = {}
             for p in self._all_parts():
                 if hasattr(p, "step_vectors"):
-                    seen.setdefault(type(p), p)
+                    # a part made of other parts names them: its vectors are theirs
+                    seen.setdefault(getattr(p, "step_vectors_key", type(p)), p)
             self._vector_makers = list(seen.values())
         out: dict = {}
         for p in self._vector_makers:
@@ -152,9 +156,17 @@ class DecoderModel:
         if self._after is None:
             self._after = self._negotiate()
         x = self.embedding.forward(ctx.ids)
+        again = x.clone() if any(e.add_input for e in self.schedule) else None   # the stream is updated in place
         carry = None
         for i, e in enumerate(self.schedule):
             block, after = self.blocks[e.layer], self._after[i]
+            if e.add_input:
+                if isinstance(carry, torch.Tensor):      # what the run before left to be added, and the embedding output
+                    carry = kernels.scaled_sum(carry, again, 1.0, 1.0)
+                elif carry is None:
+                    carry = again
+                else:
+                    raise ValueError("a schedule entry that adds the embedding output follows a block whose carry is no tensor")
             if after is None:
                 carry = block.forward(x, carry, ctx, caches[i])
             else:

@@ -106,8 +106,8 @@ def _i32(t: torch.Tensor, what: str, n: int | None = None) -> None:
 
 
 # ---------------------------------------------------------------------------------------------
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """x[t] = float(table[ids[t]]); the residual stream is float32 in every mode."""
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
+    """x[t] = float(table[ids[t]]) * scale; the residual stream is float32 in every mode."""
     _on_gpu(ids, table, out)
     _i32(ids, "ids")
     _check(table.dim() == 2 and table.is_contiguous(), "embedding table must be a contiguous [V, H] matrix")
@@ -115,7 +115,7 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = Non
     if out is None:
         out = torch.empty(T, H, dtype=torch.float32, device=table.device)
     _check(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H), "embed: bad output")
-    _call("tl_embed", _ptr(ids), _ptr(table), _code(table, "embed"), _ptr(out), T, H, V, _stream())
+    _call("tl_embed", _ptr(ids), _ptr(table), _code(table, "embed"), _ptr(out), T, H, V, ctypes.c_float(scale), _stream())
     return out
 
 
@@ -700,14 +700,16 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None,
                     q_start: torch.Tensor | None = None, ctx_start: torch.Tensor | None = None, plan=None,
                     path: str | None = None, split_keys: int | None = None,
-                    single_seqs: torch.Tensor | None = None, route_singles: bool | None = None) -> torch.Tensor:
+                    single_seqs: torch.Tensor | None = None, route_singles: bool | None = None,
+                    sink: bool = False) -> torch.Tensor:
     """Causal attention of each token over the cached keys of its sequence.
 
     ``q``: [T, >= nq*d] with the query heads in the first nq*d columns (row stride free);
     ``tables``: int32 [S, NB] page ids; ``seq_of_token``, ``pos``: int32 [T]; ``plan``: the step's
     host-side facts (``max_context``, ``max_query_len``, ``decode_only``, ``num_seqs``, ``q_lens``,
     ``starts``, ``fit_context``).  ``window`` > 0
-    limits a token at position p to keys [p - window + 1, p].  Returns [T, nq*d].
+    limits a token at position p to keys [p - window + 1, p].  ``sink`` adds one to the softmax's
+    denominator (a key of score 0 that has no value): ``p_j = exp(s_j) / (1 + sum exp(s))``.  Returns [T, nq*d].
 
     bfloat16 with a head size of 32, 64 or 128 and pages of a multiple of 8 tokens runs on the
     matrix cores; that kernel works per sequence and needs ``q_start`` [S+1], ``ctx_start`` [S]
@@ -763,7 +765,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                       _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws[:n_o]), _ptr(ws[n_o:]), T, S,
                       num_heads, num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt1,
                       -(-G // (16 * nt1)), nsplit, max(split_len // 32, 1), 0, 0, _ptr(single_seqs), len(singles), 0,
-                      _stream())
+                      int(bool(sink)), _stream())
                 skip_single = 1
         q_lens = [n for n in plan.q_lens if n > 1] if skip_single else plan.q_lens
         nt = 1 if plan.max_query_len * G <= 16 or head_dim == 256 else 2
@@ -795,14 +797,14 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             total = sum(-(-n * G // cols) for n in q_lens) + pads
             _call("tl_attention_tile32", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
                   _ptr(q_start), _ptr(ctx_start), _ptr(out), o_stride, T, S, num_heads, num_kv_heads, head_dim, page,
-                  int(window), ctypes.c_float(scale), waves, total, skip_single, _stream())
+                  int(window), ctypes.c_float(scale), waves, total, skip_single, int(bool(sink)), _stream())
             return out
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
               0 if path == "mfma-direct" else _tile16_chains(total128, num_kv_heads, path, plan.max_context), total128,
               _ptr(None), 0,
-              skip_single, _stream())
+              skip_single, int(bool(sink)), _stream())
         return out
     # The any-shape kernel tiles each sequence's tokens: it needs the first row of every sequence and the
     # most tokens one of them brings.  The engine has both; a bare call derives them from seq_of_token.
@@ -835,7 +837,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
           _ptr(q_start), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, S, max(max_query_len, 1), num_heads,
-          num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nsplit, split_len, _ptr(ws), _stream())
+          num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nsplit, split_len, _ptr(ws), int(bool(sink)), _stream())
     return out
 
 
@@ -947,6 +949,24 @@ def tanh_rows(z: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def relu_squared(z: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """``max(z, 0)^2`` of a float32 tensor, in ``out_dtype``."""
+    _on_gpu(z)
+    _check(z.dtype == torch.float32 and z.is_contiguous(), "relu_squared: input must be contiguous float32")
+    out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+    _call("tl_unary", _ptr(z), _ptr(out), _code(out, "relu_squared out"), ctypes.c_longlong(z.numel()), 1, _stream())
+    return out
+
+
+def scaled_sum(x: torch.Tensor, y: torch.Tensor, a: float, b: float) -> torch.Tensor:
+    """``a * x + b * y`` of two float32 tensors of one shape, written over ``x``."""
+    _on_gpu(x, y)
+    _check(x.dtype == y.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape,
+           "scaled_sum: two contiguous float32 tensors of one shape are needed")
+    _call("tl_scaled_sum", _ptr(x), _ptr(y), _ptr(x), ctypes.c_float(a), ctypes.c_float(b), ctypes.c_longlong(x.numel()), _stream())
+    return x
+
+
 def clamp_glu(gate_up: torch.Tensor, limit: float, alpha: float, out_dtype: torch.dtype | None = None) -> torch.Tensor:
     """For a fused [T, 2F] projection (gate columns first): ``g = min(gate, limit)``, ``u = clamp(up,
     -limit, limit)``, result ``g * sigmoid(alpha g) * (u + 1)`` [T, F]."""
@@ -963,26 +983,31 @@ def gated_group_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, 
                      out_dtype: torch.dtype) -> torch.Tensor:
     """``o`` float32 [T, N] in groups of ``group`` columns, each divided by its root mean square (eps
     inside the root), times ``weight`` [N], times ``sigmoid(gate)`` or ``silu(gate)`` (``gate`` float32
-    [T, N], rows may be strided)."""
+    [T, N], rows may be strided).  ``gate_act`` "silu_first" puts the gate ahead of the norm: ``o *
+    silu(gate)`` is what each group divides by its root mean square, then times ``weight``."""
     _on_gpu(o, weight, gate)
     T, N = o.shape
     _check(o.dtype == torch.float32 and o.stride(1) == 1 and gate.dtype == torch.float32 and gate.stride(1) == 1
            and tuple(gate.shape) == (T, N), "gated_group_norm: o and gate must be float32 [T, N]")
     _f32(weight, "gated_group_norm weight", N)
-    _check(gate_act in ("sigmoid", "silu") and group > 0 and N % group == 0, "gated_group_norm: bad group or gate")
+    _check(gate_act in _GATE_ACTS and group > 0 and N % group == 0, "gated_group_norm: bad group or gate")
     out = torch.empty(T, N, dtype=out_dtype, device=o.device)
     _call("tl_gated_group_norm", _ptr(o), o.stride(0) if T > 1 else N, _ptr(weight), _ptr(gate), gate.stride(0) if T > 1 else N,
-          _ptr(out), _code(out, "gated_group_norm out"), T, N, int(group), ctypes.c_float(eps), 0 if gate_act == "sigmoid" else 1,
+          _ptr(out), _code(out, "gated_group_norm out"), T, N, int(group), ctypes.c_float(eps), _GATE_ACTS[gate_act],
           _stream())
     return out
 
 
+_GATE_ACTS = {"sigmoid": 0, "silu": 1, "silu_first": 2}
+
+
 def _state_ptr(state: torch.Tensor, offset: int) -> tuple[ctypes.c_void_p, int]:
     """(address of element ``offset`` of slot 0, elements from one slot to the next) of a float32
-    state arena [slots, n]."""
-    _check(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous() and 0 <= offset < state.shape[1],
-           "a state arena must be contiguous float32 [slots, n]")
-    return ctypes.c_void_p(state.data_ptr() + 4 * offset), state.shape[1]
+    state arena [slots, n]; the arena may be a block of columns of a wider one (a mixer's share of the
+    state that several mixers of a layer keep side by side)."""
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and 0 <= offset < state.shape[1],
+           "a state arena must be float32 [slots, n] with a slot's values contiguous")
+    return ctypes.c_void_p(state.data_ptr() + 4 * offset), state.stride(0)
 
 
 def token_shift(h: torch.Tensor, mu: torch.Tensor, ctx, state: torch.Tensor, offset: int) -> torch.Tensor:
@@ -1105,50 +1130,70 @@ def recurrence_takes_key_dim(dk: int) -> bool:
 
 def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ctx, state: torch.Tensor, heads: int, dk: int,
                       dv: int, decay: torch.Tensor | None = None, wlog: torch.Tensor | None = None,
-                      bonus: torch.Tensor | None = None, silu_inputs: bool = False) -> torch.Tensor:
+                      bonus: torch.Tensor | None = None, silu_inputs: bool = False, steps: torch.Tensor | None = None,
+                      rate_log: torch.Tensor | None = None, step_bias: torch.Tensor | None = None,
+                      skip: torch.Tensor | None = None, share: int = 1, state_offset: int = 0) -> torch.Tensor:
     """Per sequence and head, token by token, with the state S [dk, dv] of the sequence's slot
-    (``state[slot, : heads * dk * dv]``, float32, updated in place):
+    (``state[slot, state_offset : state_offset + heads * dk * dv]``, float32, updated in place):
 
     * ``decay`` float32 [heads]: ``S <- decay_h S + k_t v_t^T``, ``o_t = S^T q_t``;
     * ``wlog`` float32 [T, heads * dk] and ``bonus`` [heads, dk]: ``o_t = (S + diag(bonus) k_t v_t^T)^T
-      q_t``, then ``S <- diag(exp(-exp(wlog_t))) S + k_t v_t^T``.
+      q_t``, then ``S <- diag(exp(-exp(wlog_t))) S + k_t v_t^T``;
+    * ``steps`` float32 [T, heads] with ``rate_log`` [heads], ``step_bias`` [heads] and ``skip`` [heads]
+      (the last two optional): ``dt = softplus(steps_t + step_bias)``, ``S <- exp(-exp(rate_log) dt) S + dt
+      k_t v_t^T``, ``o_t = S^T q_t + skip v_t``; the ``share`` consecutive heads of a group read the same
+      queries and keys (``q``, ``k`` [T, heads / share * dk]).
 
     ``q``, ``k`` [T, heads * dk] and ``v`` [T, heads * dv] are float32 and may be column blocks of a
     wider matrix; ``silu_inputs`` applies SiLU to all three on the way in.  Returns float32 [T, heads * dv]."""
-    _on_gpu(q, k, v, state, decay, wlog, bonus)
+    _on_gpu(q, k, v, state, decay, wlog, bonus, steps, rate_log, step_bias, skip)
     T = q.shape[0]
-    for name, t, n in (("q", q, heads * dk), ("k", k, heads * dk), ("v", v, heads * dv)):
+    share = int(share) if steps is not None else 1
+    _check(share >= 1 and heads % share == 0, f"linear_recurrence: {heads} heads do not share queries in groups of {share}")
+    for name, t, n in (("q", q, heads // share * dk), ("k", k, heads // share * dk), ("v", v, heads * dv)):
         _check(t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1 and tuple(t.shape) == (T, n),
                f"linear_recurrence: {name} must be float32 [T, {n}]")
-    per_token = wlog is not None
-    if per_token:
+    per_token = 2 if steps is not None else 1 if wlog is not None else 0
+    if per_token == 2:
+        _check(steps.dtype == torch.float32 and steps.dim() == 2 and steps.stride(1) == 1 and tuple(steps.shape) == (T, heads)
+               and rate_log is not None, "linear_recurrence: steps must be float32 [T, heads], with a rate per head")
+        _f32(rate_log, "linear_recurrence rate_log", heads)
+        for name, t in (("step_bias", step_bias), ("skip", skip)):
+            if t is not None:
+                _f32(t, "linear_recurrence " + name, heads)
+        wlog, decay, bonus = steps, rate_log, step_bias
+    elif per_token:
         _check(wlog.dtype == torch.float32 and wlog.stride(1) == 1 and tuple(wlog.shape) == (T, heads * dk), "linear_recurrence: bad decays")
         if bonus is not None:
             _f32(bonus, "linear_recurrence bonus", heads * dk)
     else:
         _check(decay is not None, "linear_recurrence: a decay per head or per token is needed")
         _f32(decay, "linear_recurrence decay", heads)
-    _check(heads * dk * dv <= state.shape[1], "linear_recurrence: the state of a request is too small")
-    st, stride = _state_ptr(state, 0)
+    _check(state_offset + heads * dk * dv <= state.shape[1], "linear_recurrence: the state of a request is too small")
+    st, stride = _state_ptr(state, state_offset)
     out = torch.empty(T, heads * dv, dtype=torch.float32, device=q.device)
     ld = lambda t: t.stride(0) if T > 1 else max(t.shape[1], t.stride(0))
     _call("tl_linear_recurrence", _ptr(q), ld(q), _ptr(k), ld(k), _ptr(v), ld(v), _ptr(wlog), ld(wlog) if per_token else 0,
-          _ptr(decay), _ptr(bonus), 1 if per_token else 0, st, ctypes.c_longlong(stride), _ptr(ctx.state_slots),
+          _ptr(decay), _ptr(bonus), per_token, _ptr(skip if per_token == 2 else None), share,
+          st, ctypes.c_longlong(stride), _ptr(ctx.state_slots),
           _ptr(ctx.q_start), _ptr(out), heads * dv, ctx.num_seqs, heads, dk, dv, 1 if silu_inputs else 0, _stream())
     return out
 
 
 # ---------------------------------------------------------------------------------------------
 # Routed experts
-def moe_route(logits: torch.Tensor, top: int) -> tuple[torch.Tensor, torch.Tensor]:
+def moe_route(logits: torch.Tensor, top: int, weighting: str = "softmax_top", scale: float = 1.0) -> tuple[torch.Tensor, torch.Tensor]:
     """Per row of float32 ``logits`` [T, E]: the ``top`` largest (lowest index first among equals), as
-    int32 ids [T, top], and the softmax over those alone, float32 [T, top]."""
+    int32 ids [T, top], and their weights, float32 [T, top]: the softmax over those alone
+    (``weighting`` "softmax_top"), or ``scale * sigmoid(logit)`` of each, not renormalised ("sigmoid")."""
+    _check(weighting in ("softmax_top", "sigmoid"), f"moe_route: unknown weighting {weighting!r}")
     _on_gpu(logits)
     T, E = logits.shape
     _check(logits.dtype == torch.float32 and logits.stride(1) == 1, "moe_route: logits must be float32 [T, E]")
     ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     weights = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    _call("tl_moe_route", _ptr(logits), logits.stride(0) if T > 1 else E, _ptr(ids), _ptr(weights), T, E, int(top), _stream())
+    _call("tl_moe_route", _ptr(logits), logits.stride(0) if T > 1 else E, _ptr(ids), _ptr(weights), T, E, int(top),
+          1 if weighting == "sigmoid" else 0, ctypes.c_float(scale), _stream())
     return ids, weights
 
 
@@ -1158,9 +1203,11 @@ def moe_tile_rows(pairs: int, experts: int) -> int:
 
 
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
-                limit: float, alpha: float, shared: torch.Tensor | None = None) -> torch.Tensor:
+                limit: float, alpha: float, shared: torch.Tensor | None = None, shift: float = 1.0) -> torch.Tensor:
     """``out[t] = sum_c weights[t, c] * expert_{ids[t, c]}(h[t]) (+ shared[t])`` in float32, where expert
-    e is ``down[e] @ act(gate_up[e] @ h)`` with the clamped gated activation of :func:`clamp_glu`.
+    e is ``down[e] @ act(gate_up[e] @ h)`` with the gated activation ``g' sigmoid(alpha g') (u' + shift)``,
+    ``g' = min(g, limit)``, ``u' = clamp(u, -limit, limit)`` (:func:`clamp_glu` has ``shift`` 1; an infinite
+    ``limit`` with ``alpha`` 1 and ``shift`` 0 is ``silu(g) * u``).
     ``gate_up`` [E, 2F, K] (gate rows first), ``down`` [E, N, F]; ``h`` [T, K] in the weights' dtype."""
     _on_gpu(h, gate_up, down, ids, weights, shared)
     T, K = h.shape
@@ -1181,10 +1228,102 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids:
     act = torch.empty(P, F, dtype=h.dtype, device=h.device)
     _call("tl_moe_gemm", _ptr(h), _code(h, "moe_experts input"), h.stride(0) if T > 1 else K, _ptr(gate_up),
           _code(gate_up, "moe_experts weights"), _ptr(act), _code(act, "moe_experts"), F, _ptr(order), _ptr(tiles), max_tiles, BM,
-          top, F, K, 1, ctypes.c_float(limit), ctypes.c_float(alpha), _stream())
+          top, F, K, 1, ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift), _stream())
     y = torch.empty(P, N, dtype=torch.float32, device=h.device)
     _call("tl_moe_gemm", _ptr(act), _code(act, "moe_experts"), F, _ptr(down), _code(down, "moe_experts weights"), _ptr(y), F32, N,
-          _ptr(order), _ptr(tiles), max_tiles, BM, top, N, F, 0, ctypes.c_float(0.0), ctypes.c_float(0.0), _stream())
+          _ptr(order), _ptr(tiles), max_tiles, BM, top, N, F, 0, ctypes.c_float(0.0), ctypes.c_float(0.0), ctypes.c_float(0.0),
+          _stream())
     out = torch.empty(T, N, dtype=torch.float32, device=h.device)
     _call("tl_moe_combine", _ptr(y), _ptr(weights), _ptr(shared), _ptr(out), T, N, top, _stream())
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# Mixing along the sequence one channel at a time
+CONV_MAX_TAPS = 16
+
+
+def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: torch.Tensor | None, ctx, state: torch.Tensor, offset: int,
+                act: str = "none", out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """A short causal convolution per channel: ``out[t, c] = act(bias[c] + sum_j taps[c, j] * x[t - (K - 1) +
+    j, c])`` along each sequence, the last tap the current token's.  ``x`` float32 [T, C] (may be a column
+    block of a wider matrix), ``taps`` float32 [C, K].  Inputs ahead of a sequence's first row of the step
+    are the K - 1 rows its state slot keeps at ``state[slot, offset : offset + (K - 1) * C]`` (zeros for a
+    new request); afterwards the slot keeps the sequence's last K - 1 inputs.  ``act``: "none" or "silu"."""
+    _on_gpu(x, taps, bias, state)
+    T, C = x.shape
+    K = taps.shape[1]
+    _check(x.dtype == torch.float32 and x.stride(1) == 1, "causal_conv: the input must be float32 [T, C]")
+    _check(taps.dim() == 2 and taps.shape[0] == C and 1 <= K <= CONV_MAX_TAPS, f"causal_conv: taps must be [C, up to {CONV_MAX_TAPS}]")
+    _f32(taps, "causal_conv taps")
+    if bias is not None:
+        _f32(bias, "causal_conv bias", C)
+    _check(act in ("none", "silu"), f"causal_conv: unknown activation {act!r}")
+    _check(offset + (K - 1) * C <= state.shape[1], "causal_conv: the kept inputs do not fit the state")
+    kept, stride = _state_ptr(state, offset)
+    out = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    _call("tl_causal_conv", _ptr(x), x.stride(0) if T > 1 else max(C, x.stride(0)), _ptr(taps), _ptr(bias), kept,
+          ctypes.c_longlong(stride), _ptr(ctx.state_slots), _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(out),
+          _code(out, "causal_conv out"), C, T, ctx.num_seqs, C, K, 1 if act == "silu" else 0, 1, _stream())
+    return out
+
+
+def gated_scan(gates: torch.Tensor, bias_r: torch.Tensor | None, bias_i: torch.Tensor | None,
+               u: torch.Tensor, y: torch.Tensor, lam: torch.Tensor, c: float, ctx, state: torch.Tensor, offset: int,
+               out_dtype: torch.dtype) -> torch.Tensor:
+    """The real-gated linear recurrent unit, per channel along each sequence: ``r = sigmoid(gate_r + bias_r)``,
+    ``i = sigmoid(gate_i + bias_i)``, ``a = exp(-c r softplus(lam))``, ``S <- a S + sqrt(1 - a^2) i u``, and the
+    result ``S * gelu_tanh(y)``.  ``gates`` float32 [T, blocks, 2 * W / blocks] contiguous: per block of
+    channels its gate_r, then its gate_i (what one batched product with the blocks' stacked matrices
+    leaves).  ``u``, ``y`` float32 [T, W] (column blocks of wider matrices allowed); ``S`` lives at
+    ``state[slot, offset : offset + W]``."""
+    _on_gpu(gates, bias_r, bias_i, u, y, lam, state)
+    T, W = u.shape
+    for name, t in (("u", u), ("y", y)):
+        _check(t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1 and tuple(t.shape) == (T, W),
+               f"gated_scan: {name} must be float32 [T, {W}]")
+    _check(gates.dtype == torch.float32 and gates.dim() == 3 and gates.is_contiguous() and gates.shape[0] == T
+           and gates.shape[1] * gates.shape[2] == 2 * W and gates.shape[2] % 2 == 0, "gated_scan: gates must be float32 [T, blocks, 2 W / blocks]")
+    bw = gates.shape[2] // 2
+    _f32(lam, "gated_scan lam", W)
+    for t in (bias_r, bias_i):
+        if t is not None:
+            _f32(t, "gated_scan bias", W)
+    _check(offset + W <= state.shape[1], "gated_scan: the state of a request is too small")
+    st, stride = _state_ptr(state, offset)
+    out = torch.empty(T, W, dtype=out_dtype, device=u.device)
+    ld = lambda t: t.stride(0) if T > 1 else max(W, t.stride(0))
+    _call("tl_gated_scan", _ptr(gates), ctypes.c_void_p(gates.data_ptr() + 4 * bw), 2 * W, _ptr(bias_r), _ptr(bias_i), _ptr(u),
+          ld(u), _ptr(y), ld(y), _ptr(lam), ctypes.c_float(c), st, ctypes.c_longlong(stride), _ptr(ctx.state_slots),
+          _ptr(ctx.q_start), _ptr(out), _code(out, "gated_scan out"), W, ctx.num_seqs, W, bw, 2 * bw, _stream())
+    return out
+
+
+def qk_norm_store(proj: torch.Tensor, pos: torch.Tensor, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None,
+                  eps: float, temp_coef: float, temp_every: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  slots: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """What lies between a fused q/k/v projection and attention without rotation, in one pass per token.
+    ``proj`` float32 [T, heads*dim + kv_heads*dim + kv_heads*vdim] (biases added).  Queries and keys are each
+    RMS-normed over their whole row, all heads at once (weights float32 [heads*dim] and [kv_heads*dim];
+    both None: no norm); queries are multiplied by ``1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)``
+    (``temp_every`` 0: no factor); keys and values go into the cache pages at ``slots`` (``k_cache`` [pages,
+    page, kv_heads, D], ``v_cache`` [pages, kv_heads, D, page]), heads padded with zeros to the cache's head
+    size D.  Returns the queries [T, heads * D] in ``out_dtype``."""
+    _on_gpu(proj, pos, q_weight, k_weight, k_cache, v_cache, slots)
+    T = proj.shape[0]
+    D, page = k_cache.shape[3], k_cache.shape[1]
+    _check(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1
+           and proj.shape[1] == heads * dim + kv_heads * (dim + vdim), "qk_norm_store: bad projection")
+    _check_caches(k_cache, v_cache, out_dtype, kv_heads, D, "qk_norm_store")
+    _check(D >= dim and D >= vdim, "qk_norm_store: the cache's head size is below the model's")
+    _i32(pos, "pos", T)
+    _i32(slots, "slots", T)
+    _check((q_weight is None) == (k_weight is None), "qk_norm_store: queries and keys are normed together or not at all")
+    if q_weight is not None:
+        _f32(q_weight, "qk_norm_store q weight", heads * dim)
+        _f32(k_weight, "qk_norm_store k weight", kv_heads * dim)
+    q = torch.empty(T, heads * D, dtype=out_dtype, device=proj.device)
+    _call("tl_qk_norm_store", _ptr(proj), proj.stride(0) if T > 1 else proj.shape[1], _ptr(pos), _ptr(q_weight), _ptr(k_weight),
+          ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every), _ptr(slots), _ptr(q), _ptr(k_cache), _ptr(v_cache),
+          _code(q, "qk_norm_store"), T, heads, kv_heads, dim, vdim, D, page, _stream())
+    return q

@@ -13,7 +13,7 @@ import torch
 from tensorline_amd.ops import kernels
 from tensorline_amd.parts.base import Linear, Part, TensorGetter, fuse_linears
 from tensorline_amd.parts.registry import build_part, register_mixer
-from tensorline_amd.parts.spec import CacheNeed, PartSpec, keys_and_values
+from tensorline_amd.parts.spec import CacheNeed, PartSpec, TensorDecl, keys_and_values
 
 
 @register_mixer("attention")
@@ -138,3 +138,100 @@ class PagedAttention(Part):
                                     window=self.window, q_start=ctx.q_start, ctx_start=ctx.ctx_start,
                                     plan=ctx.facts, single_seqs=ctx.extra.get("attention.single_seqs"))
         return self.o_proj(o, out_dtype=torch.float32, sink=sink)
+
+
+@register_mixer("normed_attention")
+class NormedAttention(Part):
+    """Grouped-query attention without rotation over the same paged cache, for designs that let
+    positions in by other ways.  Parameters: ``heads``, ``kv_heads``, ``dim`` (query/key size per
+    head), ``vdim`` (value size per head), ``scale`` of the scores, ``eps``;
+
+    * ``qk_norm``: queries and keys are each RMS-normed over their whole projection, all heads at
+      once, before they are split into heads (weights ``q.norm`` [heads*dim], ``k.norm``
+      [kv_heads*dim]);
+    * ``q_temp`` = {coef, every} or None: the query at position p is multiplied by
+      ``1 + coef * ln(floor((p + 1) / every) + 1)``;
+    * ``sink``: one is added to the softmax's denominator, ``p_j = exp(s_j) / (1 + sum exp(s))``: a key
+      of score 0 that has no value;
+    * ``window``: a token sees the last ``window`` keys only (0: all).
+
+    Tensors under the prefix: q, k, v (with ``.b`` where ``bias``), q.norm, k.norm, o.  Projection
+    sums, the norms and the factor are float32; what attention reads (queries, cached keys and
+    values) is in the engine's dtype.  Keys and values share one head size in the cache,
+    ``ceil16(max(dim, vdim))``: the shorter of the two is padded with zeros, which add nothing to a
+    score and come out of the weighted sum as zeros that meet zero columns of ``o``."""
+
+    def __init__(self, hidden_size, prefix, dtype, device, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 eps: float = 1e-6, bias: bool = True, qk_norm: bool = True, q_temp: dict | None = None, sink: bool = False,
+                 window: int = 0):
+        super().__init__(hidden_size, prefix, dtype, device)
+        self.heads, self.kv_heads, self.dim, self.vdim = int(heads), int(kv_heads), int(dim), int(vdim)
+        if min(self.heads, self.kv_heads, self.dim, self.vdim) <= 0 or self.heads % self.kv_heads:
+            raise ValueError(f"{prefix}: {heads} query heads of {dim} and {kv_heads} key/value heads of {vdim} do not fit")
+        self.kernel_dim = -(-max(self.dim, self.vdim) // 16) * 16
+        if not kernels.attention_takes_head_dim(self.kernel_dim):
+            raise ValueError(f"{prefix}: a head size of {max(self.dim, self.vdim)} is not served: the attention kernels "
+                             "take up to 256")
+        self.scale, self.eps, self.window = float(scale), float(eps), int(window or 0)
+        if self.scale <= 0.0:
+            raise ValueError(f"{prefix}: the score scale {scale} must be positive")
+        self.qk_norm, self.sink = bool(qk_norm), bool(sink)
+        self.temp_coef = float(q_temp["coef"]) if q_temp else 0.0
+        self.temp_every = int(q_temp["every"]) if q_temp else 0
+        if q_temp and self.temp_every <= 0:
+            raise ValueError(f"{prefix}: q_temp.every must be positive")
+        mk = lambda s, n_in, n_out, b: Linear(prefix + s, n_in, n_out, b, weight_name=prefix + s, bias_name=prefix + s + ".b")
+        self._projs = [mk("q", hidden_size, self.heads * self.dim, bias), mk("k", hidden_size, self.kv_heads * self.dim, bias),
+                       mk("v", hidden_size, self.kv_heads * self.vdim, bias)]
+        self.qkv: Linear | None = None
+        self.o_proj = mk("o", self.heads * self.vdim, hidden_size, False)
+        self.q_norm = self.k_norm = None
+
+    def tensors(self):
+        out = {}
+        for p in self._projs + [self.o_proj]:
+            out.update(p.tensors())
+        if self.qk_norm:
+            out[self.prefix + "q.norm"] = TensorDecl((self.heads * self.dim,), "one_plus_normal", 0.1, "float32")
+            out[self.prefix + "k.norm"] = TensorDecl((self.kv_heads * self.dim,), "one_plus_normal", 0.1, "float32")
+        return out
+
+    def load(self, get: TensorGetter) -> None:
+        for p in self._projs + [self.o_proj]:
+            p.load(get)
+        if self.kernel_dim != self.vdim:          # attention leaves kernel_dim columns per head: zero columns for the padding
+            w, D = self.o_proj.weight, self.kernel_dim
+            wide = w.new_zeros(w.shape[0], self.heads, D)
+            wide[:, :, :self.vdim] = w.view(w.shape[0], self.heads, self.vdim)
+            self.o_proj.weight, self.o_proj.in_features = wide.view(w.shape[0], self.heads * D), self.heads * D
+        self.qkv = fuse_linears(self.prefix + "qkv", self._projs)
+        for p in self._projs:
+            p.weight = p.bias = None
+        self.o_proj.prepare()
+        if self.qk_norm:
+            self.q_norm, self.k_norm = get(self.prefix + "q.norm"), get(self.prefix + "k.norm")
+
+    def weight_tensors(self):
+        return self.qkv.tensors_kept() + self.o_proj.tensors_kept() + [t for t in (self.q_norm, self.k_norm) if t is not None]
+
+    def library_products(self):
+        return [(self.qkv.weight, torch.float32), (self.o_proj.weight, torch.float32)]
+
+    def cache_need(self) -> CacheNeed | None:
+        return keys_and_values(self.kv_heads, self.kernel_dim, self.window)
+
+    def state_need(self):
+        return None
+
+    step_vectors = staticmethod(PagedAttention.step_vectors)
+
+    def forward(self, h, ctx, cache):
+        keys, values = cache.planes["k"], cache.planes["v"]
+        proj = self.qkv(h, out_dtype=torch.float32)
+        q = kernels.qk_norm_store(proj, ctx.pos, self.q_norm, self.k_norm, self.eps, self.temp_coef, self.temp_every,
+                                  keys, values, cache.slots, self.heads, self.kv_heads, self.dim, self.vdim, self.dtype)
+        o = kernels.paged_attention(q, keys, values, cache.tables, ctx.seq_of_token, ctx.pos, self.heads, self.kv_heads,
+                                    self.kernel_dim, self.scale, window=self.window, q_start=ctx.q_start,
+                                    ctx_start=ctx.ctx_start, plan=ctx.facts,
+                                    single_seqs=ctx.extra.get("attention.single_seqs"), sink=self.sink)
+        return self.o_proj(o, out_dtype=torch.float32)

@@ -10,8 +10,8 @@ the head that turns normed rows into logits.
   the head's product).
 
 Reference: ``x = embed_tokens(ids)`` (tensorline/paged.py:240) and ``lm_head`` on the wanted rows
-(paged.py:278-287); a tied head uses the embedding's table (tensorline/manager.py:65).  An
-embedding scale, a bias or a cap on the logits would be other kinds registered beside these.
+(paged.py:278-287); a tied head uses the embedding's table (tensorline/manager.py:65).  The
+embedding takes a scale; a bias or a cap on the logits would be other kinds registered beside these.
 """
 from __future__ import annotations
 
@@ -25,11 +25,15 @@ from tensorline_amd.parts.spec import TensorDecl
 
 @register_embedding("token_embedding")
 class TokenEmbedding(Part):
-    def __init__(self, hidden_size, prefix, dtype, device, vocab_size: int, name: str, std: float = 0.02):
+    def __init__(self, hidden_size, prefix, dtype, device, vocab_size: int, name: str, std: float = 0.02,
+                 scale: float = 1.0):
+        """``scale``: a factor on every row as it enters the stream (a head tied to the table reads the
+        table itself, without it)."""
         super().__init__(hidden_size, prefix, dtype, device)
         self.vocab_size = int(vocab_size)
         self.name = prefix + name
         self.std = float(std)
+        self.scale = float(scale)
         self.table: torch.Tensor | None = None
 
     def tensors(self):
@@ -42,7 +46,7 @@ class TokenEmbedding(Part):
         return [self.table]
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        return kernels.embed(ids, self.table)
+        return kernels.embed(ids, self.table, scale=self.scale)
 
 
 @register_head("lm_head")

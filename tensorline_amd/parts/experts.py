@@ -4,6 +4,10 @@
     those ``top`` logits alone;  out = sum_chosen weight_e * expert_e(h)  (+ shared(h))
     expert(h) = W_down (g * sigmoid(alpha g) * (u + 1)),  g = min(W_gate h, limit),  u = clamp(W_up h, +-limit)
 
+Other designs change the weights (``weighting`` "sigmoid": each chosen expert by its own score,
+``router_scale * sigmoid(z_e)``, not renormalised), leave the router without bias, or use the plain
+gated activation ``silu(g) * u`` (``activation`` "swiglu": no limit, alpha 1, nothing added to u).
+
 The experts' matrices are stacked ([experts, 2 ff, width] gate over up, [experts, width, ff]); a
 step's (token, choice) pairs are ordered by expert on the device and both products run as one
 grouped launch each (``kernels.moe_experts``), with no look at the device from the host, so the
@@ -23,16 +27,29 @@ from tensorline_amd.parts.spec import TensorDecl
 @register_feed_forward("routed_experts")
 class RoutedExperts(Part):
     """Parameters: ``experts``, ``top``, ``ff`` and ``limit`` of an expert, ``shared`` = {ff, limit} or
-    None, ``alpha`` of the gate's sigmoid.  Tensors under the prefix: router, router.b, e<i>.gate /
-    .up / .down, shared.gate / .up / .down."""
+    None, ``alpha`` of the gate's sigmoid; ``weighting`` ("softmax_top" or "sigmoid"), ``router_scale``,
+    ``router_bias``, ``activation`` ("clamped_glu" or "swiglu").  Tensors under the prefix: router,
+    router.b, e<i>.gate / .up / .down, shared.gate / .up / .down."""
 
-    def __init__(self, hidden_size, prefix, dtype, device, experts: int, top: int, ff: int, limit: float,
-                 shared: dict | None = None, alpha: float = 1.702):
+    def __init__(self, hidden_size, prefix, dtype, device, experts: int, top: int, ff: int, limit: float | None = None,
+                 shared: dict | None = None, alpha: float = 1.702, weighting: str = "softmax_top", router_scale: float = 1.0,
+                 router_bias: bool = True, activation: str = "clamped_glu"):
         super().__init__(hidden_size, prefix, dtype, device)
+        if activation not in ("clamped_glu", "swiglu") or weighting not in ("softmax_top", "sigmoid"):
+            raise ValueError(f"{prefix}: unknown activation {activation!r} or weighting {weighting!r}")
+        if activation == "swiglu":
+            limit, alpha, self.shift = float("inf"), 1.0, 0.0
+        else:
+            if limit is None:
+                raise ValueError(f"{prefix}: the clamped activation needs its limit")
+            self.shift = 1.0
+        if shared and activation != "clamped_glu":
+            raise ValueError(f"{prefix}: a shared expert comes with the clamped activation only")
+        self.weighting, self.router_scale = weighting, float(router_scale)
         self.experts, self.top, self.ff, self.limit, self.alpha = int(experts), int(top), int(ff), float(limit), float(alpha)
         if not 0 < self.top <= self.experts or self.top > 32 or self.experts > 1024:
             raise ValueError(f"{prefix}: top {self.top} of {self.experts} experts is not served (top <= 32, experts <= 1024)")
-        self.router = Linear(prefix + "router", hidden_size, self.experts, True, weight_name=prefix + "router",
+        self.router = Linear(prefix + "router", hidden_size, self.experts, bool(router_bias), weight_name=prefix + "router",
                              bias_name=prefix + "router.b")
         self.gate_up = self.down = None
         self.shared_ff = int(shared["ff"]) if shared else 0
@@ -82,9 +99,9 @@ class RoutedExperts(Part):
         return [(self.shared_gate_up.weight, self.dtype), (self.shared_down.weight, torch.float32)]
 
     def forward(self, h, ctx):
-        ids, weights = kernels.moe_route(self.router(h, out_dtype=torch.float32), self.top)
+        ids, weights = kernels.moe_route(self.router(h, out_dtype=torch.float32), self.top, self.weighting, self.router_scale)
         shared = None
         if self.shared_down is not None:
             act = kernels.clamp_glu(self.shared_gate_up(h, out_dtype=torch.float32), self.shared_limit, self.alpha, self.dtype)
             shared = self.shared_down(act, out_dtype=torch.float32)
-        return kernels.moe_experts(h, self.gate_up, self.down, ids, weights, self.limit, self.alpha, shared)
+        return kernels.moe_experts(h, self.gate_up, self.down, ids, weights, self.limit, self.alpha, shared, self.shift)

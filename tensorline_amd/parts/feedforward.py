@@ -1,4 +1,5 @@
-"""Dense feed-forward: SwiGLU, ``down(silu(gate(h)) * up(h))``, no biases.
+"""Dense feed-forwards: SwiGLU, ``down(silu(gate(h)) * up(h))``, and one without gate, ``down(act(up(h)))``;
+no biases.
 
 The reference calls the checkpoint's own module for this (tensorline/paged.py:276); the
 projection names and shapes are fixed by tensorline/manager.py:52-54 and tensorline/quant.py:25.
@@ -49,3 +50,37 @@ class SwiGLU(Part):
     def forward(self, h, ctx, sink=None, keep_shares: bool = False):
         act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.streamed)
         return self.down(act, out_dtype=torch.float32, sink=sink, keep_shares=keep_shares)
+
+
+@register_feed_forward("up_down")
+class UpDown(Part):
+    """A feed-forward without gate: ``down(act(up(h)))``, no biases.  ``activation``: "relu2", the
+    square of relu, computed in float32.  Tensors under the prefix: up, down."""
+
+    ACTIVATIONS = ("relu2",)
+
+    def __init__(self, hidden_size, prefix, dtype, device, ff: int, activation: str = "relu2"):
+        super().__init__(hidden_size, prefix, dtype, device)
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"{prefix}: unknown activation {activation!r}; known: {', '.join(self.ACTIVATIONS)}")
+        self.ff, self.activation = int(ff), activation
+        self.up = Linear(prefix + "up", hidden_size, self.ff, False, weight_name=prefix + "up")
+        self.down = Linear(prefix + "down", self.ff, hidden_size, False, weight_name=prefix + "down")
+
+    def tensors(self):
+        return {**self.up.tensors(), **self.down.tensors()}
+
+    def load(self, get: TensorGetter) -> None:
+        for lin in (self.up, self.down):
+            lin.load(get)
+            lin.prepare()
+
+    def weight_tensors(self):
+        return self.up.tensors_kept() + self.down.tensors_kept()
+
+    def library_products(self):
+        return [(self.up.weight, torch.float32), (self.down.weight, torch.float32)]
+
+    def forward(self, h, ctx):
+        act = kernels.relu_squared(self.up(h, out_dtype=torch.float32), self.dtype)
+        return self.down(act, out_dtype=torch.float32)

@@ -154,3 +154,160 @@ class WKV(Part):
         o = kernels.linear_recurrence(r, k, v, ctx, cache.state, H, d, d, wlog=wlog, bonus=self.u)
         y = kernels.gated_group_norm(o, self.norm_w, g, d, self.eps, "silu", self.dtype)
         return self.o_proj(y, out_dtype=f32)
+
+
+@register_mixer("ssd")
+class StateSpaceDuality(Part):
+    """The mixer of Mamba-2 (Dao and Gu, "Transformers are SSMs: Generalized Models and Efficient
+    Algorithms Through Structured State Space Duality").  Parameters: ``heads``, ``vdim`` (a head's
+    channels), ``state`` (N), ``groups`` (heads of a group share B and C), ``conv`` (taps),
+    ``norm_groups``, ``eps``.  With inner = heads * vdim, the input projection gives
+    [z: inner | x: inner | B: groups*N | C: groups*N | dt: heads];  x, B and C pass a causal
+    convolution per channel and SiLU;  dt = softplus(dt + dt_bias);  per head
+    S_t = exp(-exp(A_log) dt) S_(t-1) + dt B_t x_t^T,  y_t = S_t^T C_t + D x_t;  y * silu(z) is RMS-normed in
+    ``norm_groups`` equal parts, times ``norm``, and projected.  The request's slot keeps S [heads, N,
+    vdim] and, behind it, the convolution's last ``conv`` - 1 inputs.  Tensors under the prefix: in,
+    conv, conv.b, dt_bias, A_log, D, norm, o."""
+
+    def __init__(self, hidden_size, prefix, dtype, device, heads: int, vdim: int, state: int, groups: int, conv: int,
+                 norm_groups: int = 1, eps: float = 1e-6):
+        super().__init__(hidden_size, prefix, dtype, device)
+        self.heads, self.vdim, self.N, self.groups = int(heads), int(vdim), int(state), int(groups)
+        self.taps, self.norm_groups, self.eps = int(conv), int(norm_groups), float(eps)
+        _check_key_dim(prefix, self.N)
+        self.inner = self.heads * self.vdim
+        if self.groups <= 0 or self.heads % self.groups:
+            raise ValueError(f"{prefix}: {heads} heads do not split into {groups} groups")
+        if self.norm_groups <= 0 or self.inner % self.norm_groups:
+            raise ValueError(f"{prefix}: {self.inner} channels do not split into {norm_groups} parts for the norm")
+        if not 1 <= self.taps <= kernels.CONV_MAX_TAPS:
+            raise ValueError(f"{prefix}: a convolution of {conv} taps is not served (1 to {kernels.CONV_MAX_TAPS})")
+        self.conv_channels = self.inner + 2 * self.groups * self.N
+        self.proj = Linear(prefix + "in", hidden_size, 2 * self.inner + 2 * self.groups * self.N + self.heads, False,
+                           weight_name=prefix + "in")
+        self.o_proj = Linear(prefix + "o", self.inner, hidden_size, False, weight_name=prefix + "o")
+        self.conv_w = self.conv_b = self.dt_bias = self.rate_log = self.skip = self.norm_w = None
+
+    def tensors(self):
+        out = {**self.proj.tensors(), **self.o_proj.tensors()}
+        p = self.prefix
+        out[p + "conv"] = TensorDecl((self.conv_channels, self.taps), "normal", 0.3, "float32")
+        out[p + "conv.b"] = TensorDecl((self.conv_channels,), "normal", 0.1, "float32")
+        out[p + "dt_bias"] = TensorDecl((self.heads,), "normal", 1.0, "float32")
+        out[p + "A_log"] = TensorDecl((self.heads,), "normal", 1.0, "float32")
+        out[p + "D"] = TensorDecl((self.heads,), "one_plus_normal", 0.3, "float32")
+        out[p + "norm"] = TensorDecl((self.inner,), "one_plus_normal", 0.1, "float32")
+        return out
+
+    def load(self, get: TensorGetter) -> None:
+        p = self.prefix
+        for lin in (self.proj, self.o_proj):
+            lin.load(get)
+            lin.prepare()
+        self.conv_w, self.conv_b = get(p + "conv"), get(p + "conv.b")
+        self.dt_bias, self.rate_log, self.skip, self.norm_w = get(p + "dt_bias"), get(p + "A_log"), get(p + "D"), get(p + "norm")
+
+    def weight_tensors(self):
+        return self.proj.tensors_kept() + self.o_proj.tensors_kept() + [
+            self.conv_w, self.conv_b, self.dt_bias, self.rate_log, self.skip, self.norm_w]
+
+    def library_products(self):
+        return [(self.proj.weight, torch.float32), (self.o_proj.weight, torch.float32)]
+
+    def cache_need(self):
+        return None
+
+    def state_need(self):
+        return StateNeed((self.heads * self.N * self.vdim + (self.taps - 1) * self.conv_channels,), "float32")
+
+    def forward(self, h, ctx, cache):
+        inner, GN, H = self.inner, self.groups * self.N, self.heads
+        proj = self.proj(h, out_dtype=torch.float32)
+        z, steps = proj[:, :inner], proj[:, 2 * inner + 2 * GN:]
+        xbc = kernels.causal_conv(proj[:, inner:2 * inner + 2 * GN], self.conv_w, self.conv_b, ctx, cache.state,
+                                  H * self.N * self.vdim, act="silu")
+        x, B, C = xbc[:, :inner], xbc[:, inner:inner + GN], xbc[:, inner + GN:]
+        y = kernels.linear_recurrence(C, B, x, ctx, cache.state, H, self.N, self.vdim, steps=steps, rate_log=self.rate_log,
+                                      step_bias=self.dt_bias, skip=self.skip, share=H // self.groups)
+        y = kernels.gated_group_norm(y, self.norm_w, z, inner // self.norm_groups, self.eps, "silu_first", self.dtype)
+        return self.o_proj(y, out_dtype=torch.float32)
+
+
+@register_mixer("rglru")
+class RealGatedLRU(Part):
+    """The recurrent block of Griffin (De et al., "Griffin: Mixing Gated Linear Recurrences with Local
+    Attention for Efficient Language Models") around its real-gated linear recurrent unit.  Parameters:
+    ``width`` of the two branches, ``blocks`` (the gates' matrices are block-diagonal), ``conv`` (taps),
+    ``c`` (the factor in ln a = -c r softplus(lam)).  y = gelu_tanh(W_y h + b),  u = conv(W_x h + b);  in
+    each block r = sigmoid(ra u + b), i = sigmoid(ri u + b);  a = exp(-c r softplus(lam)),
+    S_t = a S_(t-1) + sqrt(1 - a^2) i u  from S = 0, the first token like every other;  result W_o (S * y).
+    The request's slot keeps S [width] and, behind it, the convolution's last ``conv`` - 1 inputs.  The
+    gates and everything behind them are float32 whatever the engine's dtype.  Tensors under the prefix:
+    y, y.b, x, x.b, conv, conv.b, ra, ra.b, ri, ri.b, lam, o."""
+
+    def __init__(self, hidden_size, prefix, dtype, device, width: int, blocks: int, conv: int, c: float = 8.0):
+        super().__init__(hidden_size, prefix, dtype, device)
+        self.width, self.blocks, self.taps, self.c = int(width), int(blocks), int(conv), float(c)
+        if self.blocks <= 0 or self.width % self.blocks:
+            raise ValueError(f"{prefix}: a width of {width} does not split into {blocks} blocks")
+        if not 1 <= self.taps <= kernels.CONV_MAX_TAPS:
+            raise ValueError(f"{prefix}: a convolution of {conv} taps is not served (1 to {kernels.CONV_MAX_TAPS})")
+        mk = lambda s, n_in, n_out, b: Linear(prefix + s, n_in, n_out, b, weight_name=prefix + s, bias_name=prefix + s + ".b")
+        self._branches = [mk("y", hidden_size, self.width, True), mk("x", hidden_size, self.width, True)]
+        self.proj: Linear | None = None
+        self.o_proj = mk("o", self.width, hidden_size, False)
+        self.conv_w = self.conv_b = self.gates = self.bias_r = self.bias_i = self.lam = None
+
+    def tensors(self):
+        out = {}
+        for lin in self._branches + [self.o_proj]:
+            out.update(lin.tensors())
+        p, bw = self.prefix, self.width // self.blocks
+        out[p + "conv"] = TensorDecl((self.width, self.taps), "normal", 0.3, "float32")
+        out[p + "conv.b"] = TensorDecl((self.width,), "normal", 0.1, "float32")
+        for s in ("ra", "ri"):
+            out[p + s] = TensorDecl((self.blocks, bw, bw), "normal", 0.2, "float32")
+            out[p + s + ".b"] = TensorDecl((self.blocks, bw), "normal", 0.5, "float32")
+        out[p + "lam"] = TensorDecl((self.width,), "normal", 1.0, "float32")
+        return out
+
+    def load(self, get: TensorGetter) -> None:
+        p = self.prefix
+        for lin in self._branches:
+            lin.load(get)
+        self.proj = fuse_linears(p + "yx", self._branches)
+        for lin in self._branches:
+            lin.weight = lin.bias = None
+        self.o_proj.load(get)
+        self.o_proj.prepare()
+        self.conv_w, self.conv_b = get(p + "conv"), get(p + "conv.b")
+        # both gates of a block as one matrix [2 bw, bw]: one batched product gives [T, blocks, r | i]
+        self.gates = torch.cat([get(p + "ra"), get(p + "ri")], dim=1).contiguous()
+        bw = self.width // self.blocks
+        self.bias_r, self.bias_i = get(p + "ra.b").reshape(-1).contiguous(), get(p + "ri.b").reshape(-1).contiguous()
+        self.lam = get(p + "lam")
+        assert tuple(self.gates.shape) == (self.blocks, 2 * bw, bw)
+
+    def weight_tensors(self):
+        return self.proj.tensors_kept() + self.o_proj.tensors_kept() + [
+            self.conv_w, self.conv_b, self.gates, self.bias_r, self.bias_i, self.lam]
+
+    def library_products(self):
+        return [(self.proj.weight, torch.float32), (self.o_proj.weight, torch.float32)]
+
+    def cache_need(self):
+        return None
+
+    def state_need(self):
+        return StateNeed((self.width + (self.taps - 1) * self.width,), "float32")
+
+    def forward(self, h, ctx, cache):
+        W, nb = self.width, self.blocks
+        bw = W // nb
+        T = h.shape[0]
+        proj = self.proj(h, out_dtype=torch.float32)                       # [y | x] with their biases
+        u = kernels.causal_conv(proj[:, W:], self.conv_w, self.conv_b, ctx, cache.state, W)
+        g = torch.empty(T, nb, 2 * bw, dtype=torch.float32, device=h.device)
+        kernels.batched_linear(u.view(T, nb, bw), self.gates, g)
+        o = kernels.gated_scan(g, self.bias_r, self.bias_i, u, proj[:, :W], self.lam, self.c, ctx, cache.state, 0, self.dtype)
+        return self.o_proj(o, out_dtype=torch.float32)

@@ -4,8 +4,9 @@ A model is a :class:`ModelSpec`.  Each layer names its parts by *kind* with thei
 constants as parameters (:class:`PartSpec`); the kinds are looked up in the registries of
 :mod:`tensorline_amd.parts.registry`.  Different layers may use different mixers and
 feed-forwards.  The order of execution is data too: ``schedule`` lists layer indices, may name a
-layer twice (its weights run twice, each run with a cache of its own), and an entry may read the
-cache another entry wrote instead of writing one itself.
+layer twice (its weights run twice, each run with a cache of its own), an entry may read the
+cache another entry wrote instead of writing one itself, and an entry may have the embedding output
+added to the stream in front of it (a stack that runs several times over, fed its input again).
 """
 from __future__ import annotations
 
@@ -55,6 +56,7 @@ class LayerSpec:
 class ScheduleEntry:
     layer: int                        # index into ModelSpec.layers
     cache_from: int | None = None     # index of the schedule entry whose cache this run reads
+    add_input: bool = False           # the embedding output is added to the stream right before this run
 
 
 @dataclass(frozen=True)

@@ -12,8 +12,8 @@ def require_gpu(device):
     return torch.device(device)
 
 
-def embed(ids, table, out=None):
-    x = table[ids.long()].to(torch.float32)
+def embed(ids, table, out=None, scale=1.0):
+    x = table[ids.long()].to(torch.float32) * scale
     if out is not None:
         out.copy_(x)
         return out
