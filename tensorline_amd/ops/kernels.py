@@ -1005,7 +1005,7 @@ def _state_ptr(state: torch.Tensor, offset: int) -> tuple[ctypes.c_void_p, int]:
     """(address of element ``offset`` of slot 0, elements from one slot to the next) of a float32
     state arena [slots, n]; the arena may be a block of columns of a wider one (a mixer's share of the
     state that several mixers of a layer keep side by side)."""
-    _check(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and 0 <= offset < state.shape[1],
+    _check(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and 0 <= offset <= state.shape[1],
            "a state arena must be float32 [slots, n] with a slot's values contiguous")
     return ctypes.c_void_p(state.data_ptr() + 4 * offset), state.stride(0)
 

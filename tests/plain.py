@@ -51,11 +51,12 @@ def rope(x: torch.Tensor, positions: torch.Tensor, theta: float, rotary_dim: int
 
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, window: int = 0,
-                     q_offset: int = 0) -> torch.Tensor:
+                     q_offset: int = 0, sink: bool = False) -> torch.Tensor:
     """q: [n, nq, d]; k, v: [ctx, nkv, d]; query i sits at position q_offset + i and sees keys
     j <= q_offset + i (reference: mask m[i, j] = j <= start + i, tensorline/paged.py:237), and with a
     window only j > q_offset + i - window.  Query head h uses key/value head h // (nq // nkv)
-    (paged.py:153-157).  softmax(q k^T * scale + mask) v, in the input dtype."""
+    (paged.py:153-157).  softmax(q k^T * scale + mask) v, in the input dtype.  ``sink``: the softmax
+    runs over one more score, 0, that has no value: one is added to the denominator."""
     n, nq, d = q.shape
     ctx, nkv, _ = k.shape
     g = nq // nkv
@@ -69,7 +70,11 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
         kh, vh = k[:, h // g, :], v[:, h // g, :]
         s = (q[:, h, :] @ kh.T) * scale
         s = s.masked_fill(~allowed, float("-inf"))
-        out[:, h, :] = torch.softmax(s, dim=-1) @ vh
+        if sink:
+            s = torch.cat((s, s.new_zeros(n, 1)), dim=-1)
+            out[:, h, :] = torch.softmax(s, dim=-1)[:, :-1] @ vh
+        else:
+            out[:, h, :] = torch.softmax(s, dim=-1) @ vh
     return out
 
 

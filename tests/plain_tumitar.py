@@ -61,8 +61,9 @@ def sink_attention(h, w, p, m: dict, eps: float, positions=None):
     v = (h @ w[p + "v"].T + w[p + "v.b"]).view(T, G, dv)
     q = rms_norm(q, w[p + "q.norm"], eps)
     k = rms_norm(k, w[p + "k.norm"], eps).view(T, G, d)
-    temp = query_temperature(pos, m["q_temp"]["coef"], m["q_temp"]["every"]).to(q.dtype)
-    q = (q * temp[:, None]).view(T, H, d)
+    if m.get("q_temp"):
+        q = q * query_temperature(pos, m["q_temp"]["coef"], m["q_temp"]["every"]).to(q.dtype)[:, None]
+    q = q.view(T, H, d)
     out = h.new_zeros(T, H, dv)
     per = H // G
     for head in range(H):
@@ -148,8 +149,26 @@ def expert_ff(h, w, p):
     return (F.silu(h @ w[p + "gate"].T) * (h @ w[p + "up"].T)) @ w[p + "down"].T
 
 
-def routed_ff(h, w, p, mlp: dict):
-    ids, weights, _ = router_choice(h, w, p, mlp)
+def routed_ff(h, w, p, mlp: dict, margins=None, forced=None):
+    """``margins``: a list that gets, per call and token, how far the last chosen expert's logit lies above
+    the best one left out, in units of the spread of the token's logits (infinite where every expert is
+    chosen).  ``forced``: an iterator of [T, top] expert ids, one per call, to use in place of the router's
+    own choice (weights are still those experts' own scores); ``margins`` then gets the regret instead: how
+    far the worst forced expert's logit lies under the last one the router would have chosen, in the same
+    units (0 where the sets agree)."""
+    ids, weights, scores = router_choice(h, w, p, mlp)
+    top = int(mlp["router"]["top"])
+    z = h @ w[p + "router"].T
+    ranked = z.sort(dim=-1, descending=True).values
+    spread = z.std(dim=-1) if z.shape[1] > 1 else torch.ones(h.shape[0], dtype=h.dtype)
+    if forced is not None:
+        ids = next(forced).long()
+        weights = scores.gather(1, ids) * float(mlp["router"]["scale"])
+        if margins is not None:
+            margins.append((ranked[:, top - 1] - z.gather(1, ids).min(dim=-1).values).clamp_min(0.0) / spread)
+    elif margins is not None:
+        margins.append((ranked[:, top - 1] - ranked[:, top]) / spread if top < ranked.shape[1]
+                       else torch.full((h.shape[0],), float("inf")))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, g in zip(ids[t].tolist(), weights[t]):
@@ -157,8 +176,8 @@ def routed_ff(h, w, p, mlp: dict):
     return out
 
 
-def feed_forward(h, w, p, mlp: dict):
-    return dense_ff(h, w, p) if mlp["kind"] == "dense" else routed_ff(h, w, p, mlp)
+def feed_forward(h, w, p, mlp: dict, margins=None, forced=None):
+    return dense_ff(h, w, p) if mlp["kind"] == "dense" else routed_ff(h, w, p, mlp, margins, forced)
 
 
 # ---- the model -----------------------------------------------------------------------------------
@@ -175,7 +194,7 @@ def run_order(cfg: dict) -> list[tuple[int, bool]]:
     return order + [(i, False) for i in range(stop, n)]
 
 
-def layer_forward(x, w, cfg: dict, i: int, state=None, positions=None):
+def layer_forward(x, w, cfg: dict, i: int, state=None, positions=None, margins=None, forced=None):
     layer, eps, p = cfg["layers"][i], float(cfg["norm"]["eps"]), f"l{i}."
     h = rms_norm(x, w[p + "norm1"], eps)
     if layer["type"] == "parallel":
@@ -184,20 +203,20 @@ def layer_forward(x, w, cfg: dict, i: int, state=None, positions=None):
         y, state = rglru_mixer(h, w, p + "mix.", layer["mixer"], state)
     x = x + y
     if layer.get("mlp") is not None:
-        x = x + feed_forward(rms_norm(x, w[p + "norm2"], eps), w, p + "mlp.", layer["mlp"])
+        x = x + feed_forward(rms_norm(x, w[p + "norm2"], eps), w, p + "mlp.", layer["mlp"], margins, forced)
     return x, state
 
 
-def forward(tokens, w, cfg: dict, return_layers: bool = False):
+def forward(tokens, w, cfg: dict, return_layers: bool = False, margins=None, forced=None):
     """Logits [T, vocab] of one sequence from its first token; with ``return_layers`` also the
-    residual stream after every layer run."""
+    residual stream after every layer run.  ``margins``, ``forced``: see ``routed_ff``."""
     ids = torch.as_tensor(tokens, dtype=torch.long)
     x0 = w["embed"][ids] * float(cfg["embedding"]["scale"])
     x, seen = x0, []
     for i, again in run_order(cfg):
         if again:
             x = x + x0
-        x, _ = layer_forward(x, w, cfg, i)
+        x, _ = layer_forward(x, w, cfg, i, margins=margins, forced=forced)
         seen.append(x)
     logits = rms_norm(x, w["final.norm"], float(cfg["norm"]["eps"])) @ w["embed"].T
     return (logits, seen) if return_layers else logits

@@ -372,11 +372,12 @@ def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
 
 
 def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None,
-                    route_singles=None, pool_pages=None, spike_at=None):
+                    route_singles=None, pool_pages=None, spike_at=None, sink=False, spike_gain=4.0, score_shift=0.0):
     """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries.
     pool_pages: the sequences' pages are the last ones of a pool of that many.  ``spike``: the key
     at position 1 (or at ``spike_at(position of the query)``, if that is a key at all) is made to
-    match its query, so that it dominates the sum if it is seen."""
+    match its query, so that it dominates the sum if it is seen.  ``score_shift``: the first dimension of
+    every key and query is set so that it takes that much off every score."""
     torch.manual_seed(seed)
     S = len(lens)
     q_lens = q_lens or [1] * S
@@ -398,6 +399,10 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
             pos.append(p)
     T = len(pos)
     q = torch.randn(T, nq * d, device=DEV).to(dtype)
+    if score_shift:
+        c = (score_shift * d ** 0.5) ** 0.5
+        kc[..., 0] = c
+        q.view(T, nq, d)[..., 0] = -c
     if spike:
         # one far key among hundreds must dominate: scale a query and a matching early key
         kflat = kc.view(-1, nkv, d)
@@ -409,7 +414,7 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
                 if not 0 <= far < lens[s]:
                     continue
             row = int(tables[s, far // bs]) * bs + far % bs
-            kflat[row] = (q[t].view(nq, d)[:nkv].float() * 4).to(dtype)
+            kflat[row] = (q[t].view(nq, d)[:nkv].float() * spike_gain).to(dtype)
     from tensorline_amd.engine.batch import StepFacts
     qs = [0]
     for ql in q_lens:
@@ -423,7 +428,7 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
                               torch.tensor(pos, dtype=torch.int32, device=DEV), nq, nkv, d, d ** -0.5, window=window,
                               q_start=torch.tensor(qs, dtype=torch.int32, device=DEV),
                               ctx_start=torch.tensor(plan.starts, dtype=torch.int32, device=DEV), plan=plan,
-                              path=path, split_keys=split_keys, single_seqs=single_seqs, route_singles=route_singles)
+                              path=path, split_keys=split_keys, single_seqs=single_seqs, route_singles=route_singles, sink=sink)
     if pool_pages:
         kc, vc, tables = kc[first:], vc[first:], tables - first
     kf, vf = kc.double().cpu().view(-1, nkv, d), vc.double().cpu().permute(0, 3, 1, 2).reshape(-1, nkv, d)
@@ -434,7 +439,7 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
         keys = torch.arange(n)
         rows = tcpu[s][keys // bs] * bs + keys % bs
         qs = q[t0:t0 + ql].double().cpu().view(ql, nq, d)
-        want[t0:t0 + ql] = plain.causal_attention(qs, kf[rows], vf[rows], d ** -0.5, window=window, q_offset=n - ql)
+        want[t0:t0 + ql] = plain.causal_attention(qs, kf[rows], vf[rows], d ** -0.5, window=window, q_offset=n - ql, sink=sink)
         t0 += ql
     return out.double().cpu().view(T, nq, d), want
 
@@ -819,3 +824,36 @@ def test_attention_short_portions_behind_long_contexts_walk_their_keys_as_two_ch
         got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, lens, q_lens, spike=True, seed=4)
         torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
         assert asked == [("tl_attention_mfma", 1)], asked
+
+
+# ---- the softmax sink: one added to the denominator, in every attention kernel ---------------------------------
+SINK_CASES = [
+    # (dtype, nq, nkv, d, page, lens, q_lens, window, path, split_keys)
+    (torch.float32, 6, 2, 48, 8, [50, 7, 130, 700], [20, 7, 1, 33], 0, "generic", None),        # any-shape kernel, portions
+    (torch.float32, 6, 2, 32, 16, [900, 3, 257], None, 0, "generic", 256),                      # its key splits and merge
+    (torch.float32, 4, 4, 16, 16, [5, 1], None, 0, "generic", None),                            # its waves sharing a tile's keys
+    (torch.bfloat16, 12, 2, 80, 16, [300, 9], [40, 9], 0, None, None),                            # a head size the matrix-core kernels do not take
+    (torch.bfloat16, 28, 4, 128, 16, [1400, 1400, 2, 129], None, 0, "mfma", 64),                  # independent waves, splits, merge
+    (torch.bfloat16, 8, 2, 64, 16, [63, 64, 65, 300], None, 0, "mfma-direct", None),              # independent waves, one run
+    (torch.bfloat16, 8, 2, 64, 16, [700, 40, 9], [300, 40, 1], 0, "mfma-tile16", None),           # tiles shared through LDS
+    (torch.bfloat16, 28, 4, 128, 16, [4200, 40], [300, 40], 0, "mfma-tile16x2", None),            # two chains of tiles
+    (torch.bfloat16, 8, 2, 64, 32, [9000], [1200], 700, "mfma-tile32", None),                     # 32 columns per wave, a window
+    (torch.bfloat16, 28, 4, 128, 16, [5000, 1, 600], [64, 1, 1], 0, None, None),                  # one-token sequences beside a portion
+]
+
+
+@pytest.mark.parametrize("case", range(len(SINK_CASES)))
+@pytest.mark.parametrize("gain", [0.0, 4.0])
+def test_attention_with_a_sink_in_every_kernel(case, gain):
+    """``p_j = exp(s_j) / (1 + sum exp(s))``.  Every score has 8 taken off (a common dimension of keys and
+    queries), so that the sink holds a visible share of a row's weight also among thousands of keys; with
+    one key made to match its query the row's maximum is large and the sink's share nearly vanishes: both
+    ends of the added term's range, in every kernel and through every merge."""
+    dtype, nq, nkv, d, bs, lens, q_lens, window, path, split = SINK_CASES[case]
+    kw = dict(window=window, seed=case, spike=gain > 0, path=path, split_keys=split, spike_gain=gain or 4.0, score_shift=8.0)
+    got, want = _attention_case(dtype, nq, nkv, d, bs, lens, q_lens, sink=True, **kw)
+    without, _ = _attention_case(dtype, nq, nkv, d, bs, lens, q_lens, sink=False, **kw)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    torch.testing.assert_close(got, want, atol=tol, rtol=tol)
+    if gain == 0:
+        assert (got - without).norm() > 0.1 * without.norm(), "the sink changed nothing where it must"

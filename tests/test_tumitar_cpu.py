@@ -1,0 +1,216 @@
+"""Tumitar without a GPU: the configuration reader, the spec and its schedule, and pins of the plain
+implementation (tests/plain_tumitar.py) that the GPU tests compare the framework with."""
+import copy
+import math
+
+import pytest
+import torch
+
+from tests import plain_tumitar as P
+from tests.tumitar_helpers import CFG_A, CFG_B, CFG_C, CONFIGS, one_layer, typed, _left, _right, _parallel, _moe
+
+
+def _weights(cfg, seed=0, dtype=torch.float64):
+    from tensorline_amd.config.registry import get_architecture
+    from tensorline_amd.models.decoder import DecoderModel
+    from tensorline_amd.weights.random_init import random_tensor
+    m = DecoderModel(get_architecture("Tumitar").build_spec(typed(cfg)), torch.float32, "cpu")
+    return {n: random_tensor(n, d, seed, "cpu").to(dtype) for n, d in m.tensor_decls().items()}, m
+
+
+# ---- configuration and spec ----------------------------------------------------------------------------
+def test_config_reads_every_size_and_round_trips():
+    from tensorline_amd.config.registry import architecture_name, get_architecture
+    cfg = typed(CFG_A)
+    assert (cfg.vocab_size, cfg.hidden_size, cfg.norm_eps, cfg.embedding_scale, cfg.loop) == (320, 96, 1e-5, 0.75, (0, 2, 2))
+    again = type(cfg).from_dict(cfg.to_dict())
+    assert again == cfg and again.to_dict() == cfg.to_dict()
+    assert get_architecture(architecture_name(CFG_A)).config_cls is type(cfg)
+
+
+@pytest.mark.parametrize("name,order", [("A", [(0, False), (1, False), (0, True), (1, False), (2, False)]),
+                                        ("B", [(0, False), (1, False), (1, True), (1, True), (2, False)]),
+                                        ("C", [(0, False), (1, False)])])
+def test_schedule_repeats_the_loop_and_marks_where_the_embedding_returns(name, order):
+    from tensorline_amd.models.tumitar import tumitar_spec
+    spec = tumitar_spec(typed(CONFIGS[name]))
+    assert [(e.layer, e.add_input) for e in spec.run_order()] == order == P.run_order(CONFIGS[name])
+    assert all(e.cache_from is None for e in spec.run_order())           # every pass has a cache of its own
+
+
+def test_a_loop_of_one_pass_and_a_loop_to_the_last_layer():
+    cfg = copy.deepcopy(CFG_A)
+    cfg["loop"] = {"start": 1, "stop": 3, "times": 1}
+    assert typed(cfg).run_order() == [(0, False), (1, False), (2, False)]
+    cfg["loop"] = {"start": 1, "stop": 3, "times": 2}
+    assert typed(cfg).run_order() == [(0, False), (1, False), (2, False), (1, True), (2, False)] == P.run_order(cfg)
+
+
+@pytest.mark.parametrize("breaker", [
+    lambda c: c["layers"][0].update(type="attention"),
+    lambda c: c["layers"][0]["mixer"]["left"].pop("kv_heads"),
+    lambda c: c["layers"][0]["mixer"]["right"].update(state=0),
+    lambda c: c["layers"][1]["mixer"].pop("blocks"),
+    lambda c: c["layers"][1]["mlp"]["router"].update(top=7),
+    lambda c: c["layers"][0]["mlp"].update(kind="glu"),
+    lambda c: c.update(loop={"start": 2, "stop": 1, "times": 2}),
+    lambda c: c.update(loop={"start": 0, "stop": 4, "times": 2}),
+    lambda c: c["norm"].pop("eps"),
+])
+def test_config_refuses_what_it_cannot_serve(breaker):
+    from tensorline_amd.config.model_config import ConfigError
+    cfg = copy.deepcopy(CFG_A)
+    breaker(cfg)
+    with pytest.raises(ConfigError):
+        typed(cfg)
+
+
+def test_parts_refuse_sizes_that_do_not_fit():
+    from tensorline_amd.models.decoder import DecoderModel
+    from tensorline_amd.models.tumitar import tumitar_spec
+    for change in (lambda m: m["right"].update(groups=3), lambda m: m["right"].update(norm_groups=5),
+                   lambda m: m["left"].update(kv_heads=3), lambda m: m["left"].update(dim=300),
+                   lambda m: m["right"].update(conv=40)):
+        cfg = copy.deepcopy(CFG_A)
+        change(cfg["layers"][0]["mixer"])
+        with pytest.raises(ValueError):
+            DecoderModel(tumitar_spec(typed(cfg)), torch.float32, "cpu")
+    cfg = copy.deepcopy(CFG_A)
+    cfg["layers"][1]["mixer"]["blocks"] = 5
+    with pytest.raises(ValueError):
+        DecoderModel(tumitar_spec(typed(cfg)), torch.float32, "cpu")
+
+
+def test_tensor_names_and_shapes_follow_the_configuration():
+    _, m = _weights(CFG_A)
+    decls = m.tensor_decls()
+    assert decls["l0.mix.left.q"].shape == (96, 96) and decls["l0.mix.left.k"].shape == (48, 96) and decls["l0.mix.left.v"].shape == (80, 96)
+    assert decls["l0.mix.left.q.norm"].shape == (96,) and decls["l0.mix.left.k.norm"].shape == (48,)
+    assert decls["l0.mix.left.o"].shape == (96, 160)
+    assert decls["l0.mix.right.in"].shape == (2 * 64 + 2 * 2 * 24 + 4, 96) and decls["l0.mix.right.conv"].shape == (64 + 96, 4)
+    assert decls["l1.mix.ra"].shape == (4, 16, 16) and decls["l1.mix.ri.b"].shape == (4, 16) and decls["l1.mix.conv"].shape == (64, 3)
+    assert decls["l1.mlp.e5.down"].shape == (96, 40) and decls["l1.mlp.router"].shape == (6, 96)
+    assert "l1.mlp.router.b" not in decls and "l2.norm2" not in decls and "head" not in decls
+    assert decls["l0.mlp.up"].shape == (136, 96) and decls["final.norm"].shape == (96,)
+    # a looped layer has one set of weights and as many states and caches as it has runs
+    assert len(m.state_needs()) == 5 and m.state_needs()[0] == m.state_needs()[2]
+    assert m.state_needs()[0].shape == (4 * 24 * 16 + 3 * (64 + 96),) and m.state_needs()[1].shape == (64 + 2 * 64,)
+
+
+# ---- pins of the plain implementation ---------------------------------------------------------------------
+def test_sink_softmax_is_a_softmax_over_one_more_score_of_zero():
+    torch.manual_seed(0)
+    m = _left(2, 1, 8, 6, scale=0.7, coef=0.0, every=1)
+    w = {"q": torch.randn(16, 10), "k": torch.randn(8, 10), "v": torch.randn(6, 10), "o": torch.eye(12),
+         "q.b": torch.randn(16), "k.b": torch.randn(8), "v.b": torch.randn(6), "q.norm": torch.ones(16), "k.norm": torch.ones(8)}
+    w = {"a." + k: v.double() for k, v in w.items()}
+    h = torch.randn(5, 10).double()
+    got = P.sink_attention(h, w, "a.", m, 1e-6)
+    q = P.rms_divide(h @ w["a.q"].T + w["a.q.b"], 1e-6).view(5, 2, 8)
+    k = P.rms_divide(h @ w["a.k"].T + w["a.k.b"], 1e-6)
+    v = h @ w["a.v"].T + w["a.v.b"]
+    for t in range(5):
+        for head in range(2):
+            s = torch.cat(((k[:t + 1] @ q[t, head]) * 0.7, torch.zeros(1).double()))
+            p = torch.softmax(s, 0)
+            assert torch.allclose(got[t, head * 6:(head + 1) * 6], p[:-1] @ v[:t + 1], atol=1e-12)
+            assert p[:-1].sum() < 1.0
+
+
+def test_query_temperature_steps_with_the_position():
+    t = P.query_temperature(torch.tensor([0, 5, 6, 7, 13, 14, 700]), 0.3, 7)
+    want = [1.0, 1.0, 1 + 0.3 * math.log(2), 1 + 0.3 * math.log(2), 1 + 0.3 * math.log(3), 1 + 0.3 * math.log(3), 1 + 0.3 * math.log(101)]
+    assert torch.allclose(t, torch.tensor(want).double(), atol=1e-12)
+
+
+@pytest.mark.parametrize("cut", [[37], [1] * 37, [5, 1, 2, 20, 9], [2, 35]])
+def test_recurrent_mixers_carry_their_state_over_any_cutting(cut):
+    """Whole sequences against portions fed one after another with the state handed on: the recurrent state
+    and the convolution's last inputs are all that a later portion needs of the earlier ones."""
+    for cfg, layer in ((CFG_A, 0), (CFG_A, 1), (CFG_B, 0), (CFG_B, 1), (CFG_B, 2)):
+        w, _ = _weights(cfg, seed=3)
+        m, p = cfg["layers"][layer], f"l{layer}.mix."
+        torch.manual_seed(1)
+        h = torch.randn(37, cfg["width"]).double()
+        if m["type"] == "parallel":
+            fn = lambda x, st: P.ssd_mixer(x, w, p + "right.", m["mixer"]["right"], 1e-6, st)
+        else:
+            fn = lambda x, st: P.rglru_mixer(x, w, p, m["mixer"], st)
+        whole, _ = fn(h, None)
+        outs, st, at = [], None, 0
+        for n in cut:
+            o, st = fn(h[at:at + n], st)
+            outs.append(o)
+            at += n
+        assert torch.allclose(torch.cat(outs), whole, atol=1e-10)
+
+
+def test_state_space_recurrence_against_its_closed_form():
+    """y_t = sum over s <= t of exp(-rate (dt_(s+1) + .. + dt_t)) dt_s (C_t . B_s) x_s + D x_t."""
+    cfg = one_layer("parallel", _parallel(_left(1, 1, 8, 8), _right(2, 6, 5, 1, conv=1, norm_groups=1)), width=24)
+    w, _ = _weights(cfg, seed=5)
+    m, p = cfg["layers"][0]["mixer"]["right"], "l0.mix.right."
+    for k in ("norm",):
+        w[p + k] = torch.ones_like(w[p + k])
+    w[p + "o"] = torch.eye(12).double().repeat(2, 1)                                   # [24, 12]: reads y back twice
+    torch.manual_seed(2)
+    h = torch.randn(9, 24).double()
+    got, _ = P.ssd_mixer(h, w, p, m, 1e-6)
+    proj = h @ w[p + "in"].T
+    z, xbc, dt = proj[:, :12], proj[:, 12:34], proj[:, 34:]
+    xbc = torch.nn.functional.silu(xbc * w[p + "conv"][:, 0] + w[p + "conv.b"])
+    x, B, C = xbc[:, :12].view(9, 2, 6), xbc[:, 12:17], xbc[:, 17:]
+    dt = torch.nn.functional.softplus(dt + w[p + "dt_bias"])
+    rate = torch.exp(w[p + "A_log"])
+    y = torch.zeros(9, 2, 6).double()
+    for t in range(9):
+        for hd in range(2):
+            for s in range(t + 1):
+                y[t, hd] += torch.exp(-rate[hd] * dt[s + 1:t + 1, hd].sum()) * dt[s, hd] * (C[t] @ B[s]) * x[s, hd]
+            y[t, hd] += w[p + "D"][hd] * x[t, hd]
+    y = P.rms_divide(y.reshape(9, 12) * torch.nn.functional.silu(z), 1e-6)
+    assert torch.allclose(got, y @ w[p + "o"].T, atol=1e-10)
+
+
+def test_gated_unit_starts_from_zero_without_a_special_first_token():
+    cfg = one_layer("rglru", {"width": 12, "blocks": 2, "conv": 1}, width=16)
+    w, _ = _weights(cfg, seed=6)
+    p = "l0.mix."
+    torch.manual_seed(4)
+    h = torch.randn(1, 16).double()
+    got, (S, _) = P.rglru_mixer(h, w, p, cfg["layers"][0]["mixer"])
+    u = (h @ w[p + "x"].T + w[p + "x.b"]) * w[p + "conv"][:, 0] + w[p + "conv.b"]
+    r = torch.sigmoid(torch.cat([u[:, :6] @ w[p + "ra"][0].T, u[:, 6:] @ w[p + "ra"][1].T], 1) + w[p + "ra.b"].reshape(1, 12))
+    i = torch.sigmoid(torch.cat([u[:, :6] @ w[p + "ri"][0].T, u[:, 6:] @ w[p + "ri"][1].T], 1) + w[p + "ri.b"].reshape(1, 12))
+    a = torch.exp(-8.0 * r * torch.nn.functional.softplus(w[p + "lam"]))
+    assert torch.allclose(S, (torch.sqrt(1 - a * a) * i * u)[0], atol=1e-12)           # not i * u: the factor holds at t = 0 too
+    assert torch.allclose(got, (S * P.gelu_tanh(h @ w[p + "y"].T + w[p + "y.b"])) @ w[p + "o"].T, atol=1e-12)
+
+
+def test_router_weights_are_the_chosen_scores_not_renormalised():
+    mlp = _moe(5, 2, 4, scale=1.5)
+    w = {"m.router": torch.tensor([[1.0, 0.0], [0.0, 1.0], [-1.0, 0.0], [2.0, 2.0], [0.5, 0.5]]).double()}
+    ids, wts, scores = P.router_choice(torch.tensor([[1.0, -1.0], [0.2, 0.1]]).double(), w, "m.", mlp)
+    assert ids.tolist() == [[0, 3], [3, 0]]
+    assert torch.allclose(wts[0], 1.5 * torch.sigmoid(torch.tensor([1.0, 0.0]).double()))
+    assert torch.allclose(wts[1], 1.5 * torch.sigmoid(torch.tensor([0.6, 0.2]).double()))
+    assert scores.shape == (2, 5)
+
+
+def test_dense_feed_forward_squares_the_relu():
+    w = {"f.up": torch.tensor([[1.0], [-1.0], [0.5]]).double(), "f.down": torch.tensor([[1.0, 10.0, 100.0]]).double()}
+    assert P.dense_ff(torch.tensor([[2.0], [-3.0]]).double(), w, "f.").flatten().tolist() == [4.0 + 100.0, 90.0]
+
+
+def test_embedding_returns_before_every_pass_but_the_first():
+    """With every mixer and feed-forward silenced (output projections zero) the stream is the embedding
+    output times the number of passes seen so far."""
+    w, _ = _weights(CFG_B, seed=1)
+    for k in list(w):
+        if k.endswith(".o") or k.endswith(".down"):
+            w[k] = torch.zeros_like(w[k])
+    toks = [3, 9, 100]
+    _, layers = P.forward(toks, w, CFG_B, return_layers=True)
+    x0 = w["embed"][toks] * 2.0
+    for run, times in enumerate([1, 1, 2, 3, 3]):
+        assert torch.allclose(layers[run], x0 * times, atol=1e-12)
