@@ -443,6 +443,46 @@ def make_dense_twin(size: str):
         tie_word_embeddings=False, max_position_embeddings=32768))
 
 
+# ---- the Tumitar design beside the dense decoder at equal size ----------------------------------------
+# Layer sizes that resemble real models of its kinds: attention heads of 128 in groups of four, a state-space
+# side as wide as the model with heads of 64 and a state of 128, a gated recurrent layer as wide as the model
+# with blocks of 128, a dense feed-forward of four widths, experts of which 6 are used.  Four layers (parallel
+# + dense, parallel + experts, rglru + dense, parallel + experts), each run once.  ``dense`` has the same width,
+# layers, vocabulary and attention heads, and a SwiGLU with the mean of the feed-forward weights a token reads.
+TUMITAR_SIZES = {
+    "w1024": dict(width=1024, heads=8, experts=32, top=6, ff=512),
+    "w2048": dict(width=2048, heads=16, experts=64, top=6, ff=1408),
+    "w4096": dict(width=4096, heads=32, experts=64, top=6, ff=2048),
+}
+
+
+def make_tumitar_config(size: str):
+    from tensorline_amd.config import TumitarConfig
+    z = TUMITAR_SIZES[size]
+    W, H = z["width"], z["heads"]
+    par = {"left": {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                    "q_temp": {"coef": 0.1, "every": 1024}},
+           "right": {"heads": W // 64, "vdim": 64, "state": 128, "groups": 2, "conv": 4, "norm_groups": 2},
+           "left_scale": 0.7, "right_scale": 0.7}
+    moe = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"], "scale": 1.0}, "expert": {"ff": z["ff"]}}
+    dense = {"kind": "dense", "ff": 4 * W}
+    layers = [{"type": "parallel", "mixer": par, "mlp": dense}, {"type": "parallel", "mixer": par, "mlp": moe},
+              {"type": "rglru", "mixer": {"width": W, "blocks": W // 128, "conv": 4}, "mlp": dense},
+              {"type": "parallel", "mixer": par, "mlp": moe}]
+    return TumitarConfig.from_dict({"architecture": "Tumitar", "vocab": HYBRID_VOCAB, "width": W, "norm": {"eps": 1e-6},
+                                    "embedding": {"scale": 1.0}, "layers": layers})
+
+
+def make_tumitar_twin(size: str):
+    from tensorline_amd.config import Qwen2Config
+    z = TUMITAR_SIZES[size]
+    inter = (2 * 2 * 4 * z["width"] + 2 * 3 * z["top"] * z["ff"]) // (4 * 3) // 128 * 128
+    return Qwen2Config.from_dict(dict(
+        architectures=["Qwen2ForCausalLM"], vocab_size=HYBRID_VOCAB, hidden_size=z["width"], intermediate_size=inter,
+        num_hidden_layers=4, num_attention_heads=z["heads"], num_key_value_heads=max(1, z["heads"] // 4), head_dim=128,
+        rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768))
+
+
 def profile_step(llm, entries_of, seed: int) -> dict:
     """Event time of every kernel of one eager step, summed per entry point (milliseconds), after a
     warm-up step of the same shape."""
@@ -471,19 +511,27 @@ def profile_step(llm, entries_of, seed: int) -> dict:
     return out
 
 
-def bench_hybrid(args) -> int:
-    """Prefill and decode throughput of the hybrid design at HYBRID_SIZES beside the dense decoder at
-    equal size, and each step's time by kernel.  One JSON line; the default benchmark is not run."""
+def bench_hybrid(args, design: str = "samovik") -> int:
+    """Prefill and decode throughput of a design at real layer sizes (``samovik``: HYBRID_SIZES, ``tumitar``:
+    TUMITAR_SIZES) beside the dense decoder at equal size, and each step's time by kernel.  One JSON line;
+    the default benchmark is not run."""
     import torch
+    table, make, make_twin, model_text = {
+        "samovik": (HYBRID_SIZES, make_hybrid_config, make_dense_twin,
+                    "Samovik layer sizes (4 layers: latent attention, lightning, wkv, latent attention) beside "
+                    "Qwen2 layers of equal width (4 layers)"),
+        "tumitar": (TUMITAR_SIZES, make_tumitar_config, make_tumitar_twin,
+                    "Tumitar layer sizes (4 layers: parallel + dense, parallel + experts, rglru + dense, parallel + experts) "
+                    "beside Qwen2 layers of equal width (4 layers)")}[design]
 
     from tensorline_amd import LLM
     from tensorline_amd.engine.batch import StepEntry
     page, tokens, batch, context = 16, args.prefill_tokens, args.batch, min(args.context, 2048)
-    sizes = [s for s in (args.hybrid_sizes.split(",") if args.hybrid_sizes else sorted(HYBRID_SIZES))]
+    sizes = [s for s in (args.hybrid_sizes.split(",") if args.hybrid_sizes else sorted(table))]
     results = {}
     for size in sizes:
         row = {}
-        for which, cfg in (("hybrid", make_hybrid_config(size)), ("dense", make_dense_twin(size))):
+        for which, cfg in (("hybrid", make(size)), ("dense", make_twin(size))):
             max_len = max(context, tokens) + 16
             llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
                       num_blocks=(batch + 1) * (-(-max_len // page)) + 8, max_num_seqs=batch, max_batched_tokens=max(2048, tokens),
@@ -520,10 +568,10 @@ def bench_hybrid(args) -> int:
         row["hybrid_over_dense"] = {"prefill": round(row["hybrid"]["prefill_tok_s"] / row["dense"]["prefill_tok_s"], 3),
                                     "decode": round(row["hybrid"]["decode_tok_s"] / row["dense"]["decode_tok_s"], 3)}
         results[size] = row
-    print(json.dumps({"metric": "hybrid_design_tok_s", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
-                      "config": {"model": "Samovik layer sizes (4 layers: latent attention, lightning, wkv, latent attention) beside "
-                                          "Qwen2 layers of equal width (4 layers)", "prefill_tokens": tokens, "decode_batch": batch,
-                                 "decode_context": context, "sizes": {k: HYBRID_SIZES[k] for k in sizes}},
+    print(json.dumps({"metric": "hybrid_design_tok_s" if design == "samovik" else design + "_design_tok_s", "unit": "tok/s",
+                      "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
+                      "config": {"model": model_text, "prefill_tokens": tokens, "decode_batch": batch,
+                                 "decode_context": context, "sizes": {k: table[k] for k in sizes}},
                       "results": results}))
     return 0
 
@@ -560,6 +608,9 @@ def main() -> int:
     ap.add_argument("--hybrid", action="store_true",
                     help="instead of the default benchmark: the hybrid design (Samovik) at real layer sizes beside the dense "
                          "decoder at equal size, prefill and decode; with --profile each step's time by kernel")
+    ap.add_argument("--tumitar", action="store_true",
+                    help="the same for the Tumitar design (attention beside a state-space mixer, gated recurrent layers, dense "
+                         "and routed feed-forwards)")
     ap.add_argument("--hybrid-sizes", default="", help="which of w1024,w2048,w4096 (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -569,6 +620,8 @@ def main() -> int:
         return bench_workload(args)
     if args.hybrid:
         return bench_hybrid(args)
+    if args.tumitar:
+        return bench_hybrid(args, "tumitar")
 
     import torch
 

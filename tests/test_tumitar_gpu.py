@@ -327,7 +327,7 @@ def test_a_state_that_hardly_decays_reaches_back_hundreds_of_tokens(dtype):
     reqs = {"first": tokens_for(cfg, 30, 8), "long": toks}
     steps = steps_whole({"first": reqs["first"]}) + steps_portions({"long": toks}, sizes=(3, 64, 2, 200, 1, 1, 50, 1))
     run_and_check(model, steps, cfg, w, reqs, dtype, "slow decay", max_tokens=512, max_requests=1)   # one slot: "long" inherits it
-    assert rel_error(P.forward(toks[300:], w, cfg)[-1].numpy(), P.forward(toks, w, cfg)[-1].numpy()) > 3 * LIMIT[dtype], \
+    assert rel_error(P.forward(toks[300:], w, cfg)[-1].numpy(), P.forward(toks, w, cfg)[-1].numpy()) > 2 * LIMIT[dtype], \
         "the first 300 tokens do not show at the end: the test would not see a lost state"
 
 
