@@ -23,22 +23,26 @@ __device__ __forceinline__ float cs_gelu_tanh(float z) {
     return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-// One thread per (token, channel).  kept: the slot's [K - 1][C] inputs, the oldest first.
+// One thread per (token, channel).  kept: the slot's [K - 1][C] inputs, the oldest first.  shift != 0 (steps in
+// which every sequence brings one token): the thread also renews what the slot keeps, each value moved one
+// place down after it has been read, the token's input last; no other thread touches that channel of that slot.
 template <typename O>
 __global__ void causal_conv_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ taps,
-                                   const float* __restrict__ bias, const float* __restrict__ kept, long long state_stride,
+                                   const float* __restrict__ bias, float* __restrict__ kept, long long state_stride,
                                    const int32_t* __restrict__ state_slots, const int32_t* __restrict__ seq_of_token,
-                                   const int32_t* __restrict__ q_start, O* __restrict__ out, int ldo, int C, int K, int act) {
+                                   const int32_t* __restrict__ q_start, O* __restrict__ out, int ldo, int C, int K, int act,
+                                   int shift) {
     const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= C) return;
     const int s = seq_of_token[t];
     const int r0 = q_start[s];
-    const float* old = kept + (size_t)state_slots[s] * state_stride;
+    float* old = kept + (size_t)state_slots[s] * state_stride;
     float acc = bias ? bias[c] : 0.f;
     for (int j = 0; j < K; ++j) {
         const int r = t - (K - 1) + j;
         const float v = r >= r0 ? x[(size_t)r * ldx + c] : old[(size_t)(r - r0 + K - 1) * C + c];
         acc += taps[(size_t)c * K + j] * v;
+        if (shift && j > 0) old[(size_t)(j - 1) * C + c] = v;
     }
     if (act == 1) acc = acc / (1.0f + expf(-acc));
     out[(size_t)t * ldo + c] = tl_from_float<O>(acc);
@@ -69,7 +73,8 @@ __global__ void causal_conv_keep_kernel(const float* __restrict__ x, int ldx, fl
 
 // x float [T, >= C] (row stride ldx); taps float [C, K]; bias float [C] or null; kept: the slots' [K - 1, C]
 // at kept + slot * state_stride; act 0: none, 1: SiLU.  out [T, >= C] float or bfloat16.  `update` != 0
-// also renews what the slots keep (a second launch, after every token of the step has read the old rows).
+// also renews what the slots keep: 1 by a second launch, after every token of the step has read the old rows;
+// 2 in the same launch, for steps in which every sequence brings exactly one token (T == S).
 extern "C" int tl_causal_conv(const float* x, int ldx, const float* taps, const float* bias, float* kept,
                               long long state_stride, const int32_t* state_slots, const int32_t* seq_of_token,
                               const int32_t* q_start, void* out, int out_dtype, int ldo, int T, int S, int C, int K, int act,
@@ -77,17 +82,19 @@ extern "C" int tl_causal_conv(const float* x, int ldx, const float* taps, const 
     TL_CHECK_ARG(T >= 0 && S >= 0 && C > 0 && K >= 1 && K <= CS_MAX_TAPS, "tl_causal_conv: bad sizes C=%d taps=%d (at most %d)", C, K, CS_MAX_TAPS);
     TL_CHECK_ARG(ldx >= C && ldo >= C && state_stride >= (long long)(K - 1) * C, "tl_causal_conv: rows or the kept inputs are too short");
     TL_CHECK_ARG(S <= 65535 && tl_ceil_div(C, 256) <= 65535, "tl_causal_conv: too many sequences or channels for one launch");
+    TL_CHECK_ARG(update != 2 || T == S, "tl_causal_conv: the one-launch form is for steps of one token per sequence");
     if (T == 0 || S == 0) return 0;
+    const int shift = update == 2 ? 1 : 0;
     dim3 block(256), grid(T, tl_ceil_div(C, 256));
     if (out_dtype == TL_F32)
         hipLaunchKernelGGL(causal_conv_kernel<float>, grid, block, 0, stream, x, ldx, taps, bias, kept, state_stride, state_slots,
-                           seq_of_token, q_start, (float*)out, ldo, C, K, act);
+                           seq_of_token, q_start, (float*)out, ldo, C, K, act, shift);
     else if (out_dtype == TL_BF16)
         hipLaunchKernelGGL(causal_conv_kernel<bf16_t>, grid, block, 0, stream, x, ldx, taps, bias, kept, state_stride, state_slots,
-                           seq_of_token, q_start, (bf16_t*)out, ldo, C, K, act);
+                           seq_of_token, q_start, (bf16_t*)out, ldo, C, K, act, shift);
     else return tl_fail("tl_causal_conv: unknown dtype %d", out_dtype);
     TL_CHECK_LAUNCH("tl_causal_conv");
-    if (update && K > 1) {
+    if (update == 1 && K > 1) {
         hipLaunchKernelGGL(causal_conv_keep_kernel, dim3(tl_ceil_div(C, 256), S), block, 0, stream, x, ldx, kept, state_stride,
                            state_slots, q_start, C, K);
         TL_CHECK_LAUNCH("tl_causal_conv keep");
@@ -95,52 +102,94 @@ extern "C" int tl_causal_conv(const float* x, int ldx, const float* taps, const 
     return 0;
 }
 
-// One thread per (sequence, channel) walks the sequence's rows; the operands of the next GS_AHEAD tokens
-// are on their way in registers meanwhile.
-#define GS_AHEAD 4
+// A work-group of sixteen waves owns GS_CH channels of one sequence and takes its rows in tiles of GS_TT tokens.
+// What does not depend on the state (the gates, a, the input's factor sqrt(1 - a^2) i u, the other branch's
+// gelu) is computed by all threads, an element each at a time, and left in LDS; then the first GS_CH threads
+// walk the tile, one multiply-add per token and channel, and write the results.  The raw operands of the next
+// tile are on their way in registers meanwhile, and LDS has two buffers, so the walk of one tile and the
+// element-wise work of the next overlap.  Every element is computed by the same instructions wherever its
+// token falls in a tile or a step.  The element-wise work is the larger part (five transcendental functions per
+// element), which is why a work-group has few channels and many waves: at 2,048 channels there are 128
+// work-groups to spread over the GPU, each with four waves per SIMD to hide the functions' latencies.
+#define GS_CH 16
+#define GS_TT 64
+#define GS_THREADS 1024
+#define GS_PER (GS_CH * GS_TT / GS_THREADS)
 template <typename O>
-__global__ __launch_bounds__(64) void gated_scan_kernel(
+__global__ __launch_bounds__(GS_THREADS) void gated_scan_kernel(
     const float* __restrict__ gr, const float* __restrict__ gi, int ldg, const float* __restrict__ br,
     const float* __restrict__ bi, const float* __restrict__ u, int ldu, const float* __restrict__ y, int ldy,
     const float* __restrict__ lam, float c, float* __restrict__ state, long long state_stride,
     const int32_t* __restrict__ state_slots, const int32_t* __restrict__ q_start, O* __restrict__ out, int ldo, int W,
     int bw, int bstride) {
-    const int s = blockIdx.y, ch = blockIdx.x * blockDim.x + threadIdx.x;
-    if (ch >= W) return;
-    const int gcol = (ch / bw) * bstride + ch % bw;       // where the channel's gates lie in a row of gr and gi
+    __shared__ float as[2][GS_TT][GS_CH], bs[2][GS_TT][GS_CH], gs[2][GS_TT][GS_CH];
+    const int s = blockIdx.y, ch0 = blockIdx.x * GS_CH, tid = threadIdx.x;
     const int r0 = q_start[s], r1 = q_start[s + 1];
     if (r1 <= r0) return;
-    float* st = state + (size_t)state_slots[s] * state_stride + ch;
-    float S = *st;
-    const float rate = c * cs_softplus(lam[ch]);
-    const float b_r = br ? br[ch] : 0.f, b_i = bi ? bi[ch] : 0.f;
-    float a_r[GS_AHEAD], a_i[GS_AHEAD], a_u[GS_AHEAD], a_y[GS_AHEAD];
+    // this thread's elements of a tile: channel ch0 + tid % GS_CH of tokens tid / GS_CH + k * (GS_THREADS / GS_CH)
+    const int mc = tid % GS_CH, mt = tid / GS_CH, ch = ch0 + mc;
+    const bool ch_ok = ch < W;
+    const int gcol = ch_ok ? (ch / bw) * bstride + ch % bw : 0;   // where the channel's gates lie in a row of gr and gi
+    const float rate = ch_ok ? c * cs_softplus(lam[ch]) : 0.f;
+    const float b_r = (br && ch_ok) ? br[ch] : 0.f, b_i = (bi && ch_ok) ? bi[ch] : 0.f;
+    float v_r[GS_PER], v_i[GS_PER], v_u[GS_PER], v_y[GS_PER];
     auto fetch = [&](int t0) {
 #pragma unroll
-        for (int k = 0; k < GS_AHEAD; ++k) {
-            const int t = t0 + k < r1 ? t0 + k : r1 - 1;
-            a_r[k] = gr[(size_t)t * ldg + gcol];
-            a_i[k] = gi[(size_t)t * ldg + gcol];
-            a_u[k] = u[(size_t)t * ldu + ch];
-            a_y[k] = y[(size_t)t * ldy + ch];
+        for (int k = 0; k < GS_PER; ++k) {
+            const int t = t0 + mt +  k * (GS_THREADS / GS_CH);
+            const bool ok = ch_ok && t < r1;
+            v_r[k] = ok ? gr[(size_t)t * ldg + gcol] : 0.f;
+            v_i[k] = ok ? gi[(size_t)t * ldg + gcol] : 0.f;
+            v_u[k] = ok ? u[(size_t)t * ldu + ch] : 0.f;
+            v_y[k] = ok ? y[(size_t)t * ldy + ch] : 0.f;
         }
     };
-    fetch(r0);
-    for (int t0 = r0; t0 < r1; t0 += GS_AHEAD) {
-        float c_r[GS_AHEAD], c_i[GS_AHEAD], c_u[GS_AHEAD], c_y[GS_AHEAD];
+    auto stash = [&](int buf) {
 #pragma unroll
-        for (int k = 0; k < GS_AHEAD; ++k) c_r[k] = a_r[k], c_i[k] = a_i[k], c_u[k] = a_u[k], c_y[k] = a_y[k];
-        if (t0 + GS_AHEAD < r1) fetch(t0 + GS_AHEAD);
-#pragma unroll
-        for (int k = 0; k < GS_AHEAD; ++k) {
-            if (t0 + k >= r1) break;
-            const float r = cs_sigmoid(c_r[k] + b_r), i = cs_sigmoid(c_i[k] + b_i);
+        for (int k = 0; k < GS_PER; ++k) {
+            const int tt = mt +  k * (GS_THREADS / GS_CH);
+            const float r = cs_sigmoid(v_r[k] + b_r), i = cs_sigmoid(v_i[k] + b_i);
             const float a = expf(-rate * r);
-            S = a * S + sqrtf(1.0f - a * a) * i * c_u[k];
-            out[(size_t)(t0 + k) * ldo + ch] = tl_from_float<O>(S * cs_gelu_tanh(c_y[k]));
+            as[buf][tt][mc] = a;
+            bs[buf][tt][mc] = sqrtf(1.0f - a * a) * i * v_u[k];
+            gs[buf][tt][mc] = cs_gelu_tanh(v_y[k]);
         }
+    };
+    float* st = state + (size_t)state_slots[s] * state_stride + ch0 + tid;     // used by the walkers (tid < GS_CH) only
+    const bool walker = tid < GS_CH && ch0 + tid < W;
+    float S = walker ? *st : 0.f;
+    fetch(r0);
+    stash(0);
+    __syncthreads();
+    int cur = 0;
+    for (int t0 = r0; t0 < r1; t0 += GS_TT) {
+        const int n = min(GS_TT, r1 - t0);
+        const bool more = t0 + GS_TT < r1;
+        if (more) fetch(t0 + GS_TT);
+        if (walker) {
+            // eight tokens' factors are read from LDS at once, so that only the multiply-adds wait for each other
+            for (int tt0 = 0; tt0 < n; tt0 += 8) {
+                float a8[8], b8[8], g8[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    a8[k] = as[cur][tt0 + k][tid];
+                    b8[k] = bs[cur][tt0 + k][tid];
+                    g8[k] = gs[cur][tt0 + k][tid];
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    if (tt0 + k < n) {
+                        S = a8[k] * S + b8[k];
+                        out[(size_t)(t0 + tt0 + k) * ldo + ch0 + tid] = tl_from_float<O>(S * g8[k]);
+                    }
+                }
+            }
+        }
+        if (more) stash(cur ^ 1);
+        __syncthreads();
+        cur ^= 1;
     }
-    *st = S;
+    if (walker) *st = S;
 }
 
 // gr, gi float (row stride ldg): the gates before their bias and sigmoid, channel ch at column (ch / bw) *
@@ -156,7 +205,7 @@ extern "C" int tl_gated_scan(const float* gr, const float* gi, int ldg, const fl
                  "tl_gated_scan: gates in blocks of %d channels %d apart do not fit rows of %d", bw, bstride, ldg);
     TL_CHECK_ARG(S <= 65535, "tl_gated_scan: too many sequences for one launch");
     if (S == 0) return 0;
-    dim3 grid(tl_ceil_div(W, 64), S), block(64);
+    dim3 grid(tl_ceil_div(W, GS_CH), S), block(GS_THREADS);
     if (out_dtype == TL_F32)
         hipLaunchKernelGGL(gated_scan_kernel<float>, grid, block, 0, stream, gr, gi, ldg, br, bi, u, ldu, y, ldy, lam, c, state,
                            state_stride, state_slots, q_start, (float*)out, ldo, W, bw, bstride);

@@ -140,37 +140,34 @@ extern "C" int tl_clamp_glu(const void* gu, int in_dtype, void* out, int out_dty
 // o float [T, N] in groups of `group` columns (a head, or the whole row): every group is divided by
 // its root mean square (eps inside the root), times weight[c], times the gate: sigmoid(gate) for
 // gate_act 0, silu(gate) for 1.  gate_act 2 puts the gate first: o * silu(gate) is what is divided by
-// its root mean square, then times weight[c].  gate float [T, ldg].  One wave per group.
+// its root mean square, then times weight[c].  gate float [T, ldg].  One work-group per (token, group).
 template <typename O>
 __global__ void gated_group_norm_kernel(const float* __restrict__ o, int ldo, const float* __restrict__ weight,
                                         const float* __restrict__ gate, int ldg, O* __restrict__ out, int N, int group,
                                         float eps, int gate_act) {
-    const int t = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-    const int groups = N / group;
-    for (int g = wave; g < groups; g += nwaves) {
-        const float* row = o + (size_t)t * ldo + g * group;
-        const float* grow = gate + (size_t)t * ldg + g * group;
-        float ss = 0.f;
-        if (gate_act == 2) {
-            for (int c = lane; c < group; c += 64) {
-                const float v = row[c] * pw_silu(grow[c]);
-                ss += v * v;
-            }
-        } else {
-            for (int c = lane; c < group; c += 64) ss += row[c] * row[c];
+    __shared__ float red[16];
+    const int t = blockIdx.x, g = blockIdx.y;
+    const float* row = o + (size_t)t * ldo + g * group;
+    const float* grow = gate + (size_t)t * ldg + g * group;
+    float ss = 0.f;
+    if (gate_act == 2) {
+        for (int c = threadIdx.x; c < group; c += blockDim.x) {
+            const float v = row[c] * pw_silu(grow[c]);
+            ss += v * v;
         }
-        ss = tl_wave_sum(ss);
-        const float rstd = 1.0f / sqrtf(ss / (float)group + eps);
-        for (int c = lane; c < group; c += 64) {
-            const int n = g * group + c;
-            const float z = grow[c];
-            if (gate_act == 2) {
-                out[(size_t)t * N + n] = tl_from_float<O>(row[c] * pw_silu(z) * rstd * weight[n]);
-            } else {
-                const float gv = gate_act == 0 ? pw_sigmoid(z) : pw_silu(z);
-                out[(size_t)t * N + n] = tl_from_float<O>(row[c] * rstd * weight[n] * gv);
-            }
+    } else {
+        for (int c = threadIdx.x; c < group; c += blockDim.x) ss += row[c] * row[c];
+    }
+    ss = tl_block_sum(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)group + eps);
+    for (int c = threadIdx.x; c < group; c += blockDim.x) {
+        const int n = g * group + c;
+        const float z = grow[c];
+        if (gate_act == 2) {
+            out[(size_t)t * N + n] = tl_from_float<O>(row[c] * pw_silu(z) * rstd * weight[n]);
+        } else {
+            const float gv = gate_act == 0 ? pw_sigmoid(z) : pw_silu(z);
+            out[(size_t)t * N + n] = tl_from_float<O>(row[c] * rstd * weight[n] * gv);
         }
     }
 }
@@ -180,7 +177,8 @@ extern "C" int tl_gated_group_norm(const float* o, int ldo, const float* weight,
     TL_CHECK_ARG(T >= 0 && N > 0 && group > 0 && N % group == 0 && ldo >= N && ldg >= N, "tl_gated_group_norm: bad sizes");
     if (T == 0) return 0;
     const int groups = N / group;
-    dim3 grid(T), block(64 * (groups < 4 ? groups : 4));
+    TL_CHECK_ARG(groups <= 65535, "tl_gated_group_norm: %d groups are more than a launch takes", groups);
+    dim3 grid(T, groups), block(group >= 256 ? 256 : 64 * tl_ceil_div(group, 64));
     if (out_dtype == TL_F32)
         hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, 0, stream, o, ldo, weight, gate, ldg, (float*)out, N, group, eps, gate_act);
     else if (out_dtype == TL_BF16)

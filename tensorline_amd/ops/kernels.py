@@ -1264,7 +1264,8 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: torch.Tensor | None, 
     out = torch.empty(T, C, dtype=out_dtype, device=x.device)
     _call("tl_causal_conv", _ptr(x), x.stride(0) if T > 1 else max(C, x.stride(0)), _ptr(taps), _ptr(bias), kept,
           ctypes.c_longlong(stride), _ptr(ctx.state_slots), _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(out),
-          _code(out, "causal_conv out"), C, T, ctx.num_seqs, C, K, 1 if act == "silu" else 0, 1, _stream())
+          _code(out, "causal_conv out"), C, T, ctx.num_seqs, C, K, 1 if act == "silu" else 0,
+          2 if ctx.facts.decode_only and T == ctx.num_seqs else 1, _stream())
     return out
 
 
