@@ -151,8 +151,8 @@ def expert_ff(h, w, p):
 
 def routed_ff(h, w, p, mlp: dict, margins=None, forced=None):
     """``margins``: a list that gets, per call and token, how far the last chosen expert's logit lies above
-    the best one left out, in units of the spread of the token's logits (infinite where every expert is
-    chosen).  ``forced``: an iterator of [T, top] expert ids, one per call, to use in place of the router's
+    the best one left out, in units of the root mean square of the token's logits (infinite where every
+    expert is chosen).  ``forced``: an iterator of [T, top] expert ids, one per call, to use in place of the router's
     own choice (weights are still those experts' own scores); ``margins`` then gets the regret instead: how
     far the worst forced expert's logit lies under the last one the router would have chosen, in the same
     units (0 where the sets agree)."""
@@ -160,7 +160,7 @@ def routed_ff(h, w, p, mlp: dict, margins=None, forced=None):
     top = int(mlp["router"]["top"])
     z = h @ w[p + "router"].T
     ranked = z.sort(dim=-1, descending=True).values
-    spread = z.std(dim=-1) if z.shape[1] > 1 else torch.ones(h.shape[0], dtype=h.dtype)
+    spread = z.pow(2).mean(dim=-1).sqrt()                     # the size of the token's logits (their root mean square)
     if forced is not None:
         ids = next(forced).long()
         weights = scores.gather(1, ids) * float(mlp["router"]["scale"])

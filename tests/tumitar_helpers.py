@@ -121,3 +121,42 @@ def run_steps_with_routes(model, steps, page_size: int = 16, max_tokens: int = 5
     finally:
         kernels.moe_route = route
     return got, {rid: [torch.cat(run) for run in runs] for rid, runs in routes.items()}
+
+
+def random_config(rng) -> dict:
+    """A configuration drawn from ``rng`` (a ``random.Random``): one to four layers of either kind in any
+    order, sizes that are and are not multiples of 8 or 16, every head grouping, one to five taps, every kind
+    of feed-forward, with or without a loop."""
+    def divisor(n):
+        return rng.choice([d for d in range(1, n + 1) if n % d == 0])
+
+    def mlp():
+        kind = rng.choice(["none", "dense", "moe", "moe"])
+        if kind == "none":
+            return None
+        if kind == "dense":
+            return _dense(rng.choice([7, 24, 50, 136, 200]))
+        experts = rng.randint(1, 9)
+        return _moe(experts, rng.randint(1, experts), rng.choice([8, 20, 36, 64]), scale=rng.choice([0.5, 1.0, 2.5]))
+
+    layers = []
+    for _ in range(rng.randint(1, 4)):
+        if rng.random() < 0.6:
+            heads = rng.choice([1, 2, 3, 4, 6, 8])
+            left = _left(heads, divisor(heads), rng.choice([8, 16, 20, 24, 32, 40, 64, 128]), rng.choice([8, 12, 16, 32, 48, 64, 128]),
+                         scale=rng.choice([0.05, 0.125, 0.3]), coef=rng.choice([-0.1, 0.0, 0.3]), every=rng.choice([1, 2, 5, 16, 64]))
+            rh = rng.choice([1, 2, 3, 4, 6])
+            right = _right(rh, rng.choice([4, 8, 10, 16, 24, 64]), rng.choice([4, 8, 12, 16, 32, 64, 100]), divisor(rh),
+                           conv=rng.randint(1, 5), norm_groups=divisor(rh))
+            layers.append({"type": "parallel", "mixer": _parallel(left, right, rng.choice([0.3, 0.8, 1.0]), rng.choice([0.5, 1.0, 1.7])),
+                           "mlp": mlp()})
+        else:
+            blocks = rng.randint(1, 5)
+            layers.append({"type": "rglru", "mixer": {"width": blocks * rng.choice([4, 8, 10, 16, 30]), "blocks": blocks,
+                                                      "conv": rng.randint(1, 5)}, "mlp": mlp()})
+    cfg = {"architecture": "Tumitar", "vocab": rng.randint(50, 400), "width": rng.choice([24, 36, 50, 64, 72, 100, 128, 200]),
+           "norm": {"eps": rng.choice([1e-5, 1e-6])}, "embedding": {"scale": rng.choice([0.5, 1.0, 3.0])}, "layers": layers}
+    if rng.random() < 0.6:
+        start = rng.randrange(len(layers))
+        cfg["loop"] = {"start": start, "stop": rng.randint(start + 1, len(layers)), "times": rng.randint(1, 3)}
+    return cfg
