@@ -472,7 +472,7 @@ extern "C" int tl_attention_wide(const void* q, const void* k_cache, int dtype, 
 //   * k goes into the cache at `slot` ([pages, page, G, D], zeros from d to D), v with a page's tokens
 //     innermost ([pages, G, D, page], zeros from dv to D).
 template <typename T>
-__global__ __launch_bounds__(256) void qk_norm_store_kernel(
+__global__ __launch_bounds__(1024) void qk_norm_store_kernel(
     const float* __restrict__ proj, int ldp, const int32_t* __restrict__ pos, const float* __restrict__ wq,
     const float* __restrict__ wk, float eps, float coef, int every, const int32_t* __restrict__ slots,
     T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int d, int dv, int D, int page) {
@@ -529,7 +529,8 @@ extern "C" int tl_qk_norm_store(const float* proj, int ldp, const int32_t* pos, 
     TL_CHECK_ARG(ldp >= H * d + G * d + G * dv, "tl_qk_norm_store: the projection's rows are too short");
     TL_CHECK_ARG((wq == nullptr) == (wk == nullptr), "tl_qk_norm_store: queries and keys are normed together or not at all");
     if (T == 0) return 0;
-    dim3 grid(T), block(256);
+    // few tokens (decode steps): a token's columns over more threads, since nothing else fills the GPU
+    dim3 grid(T), block(T <= 64 && H * D >= 1024 ? 1024 : 256);
     if (dtype == TL_F32)
         hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, 0, stream, proj, ldp, pos, wq, wk, eps, coef, every, slots,
                            (float*)q_out, (float*)k_cache, (float*)v_cache, H, G, d, dv, D, page);

@@ -215,7 +215,7 @@ class NormedAttention(Part):
         return self.qkv.tensors_kept() + self.o_proj.tensors_kept() + [t for t in (self.q_norm, self.k_norm) if t is not None]
 
     def library_products(self):
-        return [(self.qkv.weight, torch.float32), (self.o_proj.weight, torch.float32)]
+        return [(lin.weight, torch.float32) for lin in (self.qkv, self.o_proj) if lin.weight is not None]
 
     def cache_need(self) -> CacheNeed | None:
         return keys_and_values(self.kv_heads, self.kernel_dim, self.window)
@@ -225,9 +225,17 @@ class NormedAttention(Part):
 
     step_vectors = staticmethod(PagedAttention.step_vectors)
 
+    def input_linear(self) -> Linear:
+        """The product this mixer applies to its input first (float32 out).  A part that runs it beside
+        another mixer may fuse the two products and hand each its columns (``forward_projected``)."""
+        return self.qkv
+
     def forward(self, h, ctx, cache):
+        return self.forward_projected(self.qkv(h, out_dtype=torch.float32), ctx, cache)
+
+    def forward_projected(self, proj, ctx, cache):
+        """``proj`` float32 [T, q | k | v] with the biases added; rows may be strided."""
         keys, values = cache.planes["k"], cache.planes["v"]
-        proj = self.qkv(h, out_dtype=torch.float32)
         q = kernels.qk_norm_store(proj, ctx.pos, self.q_norm, self.k_norm, self.eps, self.temp_coef, self.temp_every,
                                   keys, values, cache.slots, self.heads, self.kv_heads, self.dim, self.vdim, self.dtype)
         o = kernels.paged_attention(q, keys, values, cache.tables, ctx.seq_of_token, ctx.pos, self.heads, self.kv_heads,

@@ -212,7 +212,7 @@ class StateSpaceDuality(Part):
             self.conv_w, self.conv_b, self.dt_bias, self.rate_log, self.skip, self.norm_w]
 
     def library_products(self):
-        return [(self.proj.weight, torch.float32), (self.o_proj.weight, torch.float32)]
+        return [(lin.weight, torch.float32) for lin in (self.proj, self.o_proj) if lin.weight is not None]
 
     def cache_need(self):
         return None
@@ -220,9 +220,17 @@ class StateSpaceDuality(Part):
     def state_need(self):
         return StateNeed((self.heads * self.N * self.vdim + (self.taps - 1) * self.conv_channels,), "float32")
 
+    def input_linear(self) -> Linear:
+        """The product this mixer applies to its input first (float32 out).  A part that runs it beside
+        another mixer may fuse the two products and hand each its columns (``forward_projected``)."""
+        return self.proj
+
     def forward(self, h, ctx, cache):
+        return self.forward_projected(self.proj(h, out_dtype=torch.float32), ctx, cache)
+
+    def forward_projected(self, proj, ctx, cache):
+        """``proj`` float32 [T, z | x | B | C | dt]; rows may be strided."""
         inner, GN, H = self.inner, self.groups * self.N, self.heads
-        proj = self.proj(h, out_dtype=torch.float32)
         z, steps = proj[:, :inner], proj[:, 2 * inner + 2 * GN:]
         xbc = kernels.causal_conv(proj[:, inner:2 * inner + 2 * GN], self.conv_w, self.conv_b, ctx, cache.state,
                                   H * self.N * self.vdim, act="silu")
