@@ -839,6 +839,9 @@ SINK_CASES = [
     (torch.bfloat16, 28, 4, 128, 16, [4200, 40], [300, 40], 0, "mfma-tile16x2", None),            # two chains of tiles
     (torch.bfloat16, 8, 2, 64, 32, [9000], [1200], 700, "mfma-tile32", None),                     # 32 columns per wave, a window
     (torch.bfloat16, 28, 4, 128, 16, [5000, 1, 600], [64, 1, 1], 0, None, None),                  # one-token sequences beside a portion
+    (torch.bfloat16, 4, 2, 256, 16, [900, 70, 3], [200, 1, 3], 0, None, None),                    # a head size of 256: one column tile per wave
+    (torch.bfloat16, 4, 1, 256, 16, [2500, 300], None, 0, "mfma", 128),                           # the same, decoded, with splits
+    (torch.bfloat16, 6, 3, 192, 16, [700, 20], [100, 1], 0, None, None),                          # 192: the any-shape kernel
 ]
 
 
