@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from tests import plain_tumitar as P
-from tests.tumitar_helpers import CFG_A, CFG_B, CFG_C, CONFIGS, one_layer, typed, _left, _right, _parallel, _moe
+from tests.tumitar_helpers import CFG_A, CFG_B, CONFIGS, one_layer, typed, _left, _right, _parallel, _moe
 
 
 def _weights(cfg, seed=0, dtype=torch.float64):

@@ -13,7 +13,7 @@ from tests import plain_tumitar as P
 from tests.helpers import steps_portions, steps_prefill_then_decode, steps_whole
 from tests.samovik_helpers import LIMIT, rel_error, run_steps
 from tests.test_samovik_gpu import mixed_steps
-from tests.tumitar_helpers import (CFG_A, CFG_B, CFG_C, CONFIGS, build, one_layer, run_steps_with_routes, typed, _dense, _left, _moe,
+from tests.tumitar_helpers import (CFG_A, CFG_B, CONFIGS, build, one_layer, run_steps_with_routes, typed, _dense, _left, _moe,
                                    _parallel, _right)
 
 pytestmark = pytest.mark.gpu
