@@ -98,6 +98,9 @@ struct TlNormArgs {
     int a_ld;
     float* ss_out;             // [tiles, ss_out_ld]: row `tile` gets the tile's sums of resid^2, one per row
     int ss_out_ld;
+    // activation of a plain product's output, after the bias (the few-row kernel; no sink with it):
+    // 0 none, 1 the square of relu
+    int act;
 };
 
 // ---- host side -----------------------------------------------------------------------------

@@ -312,6 +312,10 @@ __global__ __launch_bounds__(MODE == MODE_SWIGLU ? 256 : 512) void gemm_skinny_k
         } else if (bias) {
             v += bias[n];
         }
+        if (MODE == MODE_PLAIN && na.act == 1) {
+            const float p = fmaxf(v, 0.f);
+            v = p * p;
+        }
         C[(size_t)m * ldc + n] = tl_from_float<TO>(v);
     }
     if (sink) {
@@ -370,6 +374,8 @@ static int check_norm(const TlNormArgs* norm, TlNormArgs* na, int M, int N, bool
     if (na->ss_in)
         TL_CHECK_ARG(na->ss_n > 0 && na->ss_ld >= M && na->dim > 0.f && na->eps >= 0.f,
                      "tl_gemm_skinny: bad owed-norm arguments (partials %d, stride %d)", na->ss_n, na->ss_ld);
+    TL_CHECK_ARG(na->act == 0 || (na->act == 1 && sink_allowed && !na->resid),
+                 "tl_gemm_skinny: activation %d is not one a plain product without a sink applies", na->act);
     if (na->resid) {
         TL_CHECK_ARG(sink_allowed, "tl_gemm_skinny: only a plain product can add into the residual");
         TL_CHECK_ARG(na->next_weight && na->a_out && na->ss_out && na->resid_ld >= N && na->a_ld >= N &&

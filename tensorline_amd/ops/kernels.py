@@ -240,7 +240,7 @@ class _NormArgs(ctypes.Structure):
                 ("dim", ctypes.c_float), ("eps", ctypes.c_float),
                 ("resid", ctypes.c_void_p), ("resid_ld", ctypes.c_int), ("next_weight", ctypes.c_void_p),
                 ("a_out", ctypes.c_void_p), ("a_ld", ctypes.c_int), ("ss_out", ctypes.c_void_p),
-                ("ss_out_ld", ctypes.c_int)]
+                ("ss_out_ld", ctypes.c_int), ("act", ctypes.c_int)]
 
 
 def can_defer_norm(num_rows: int, dtype: torch.dtype) -> bool:
@@ -280,13 +280,36 @@ def _norm_args(owed: NormedRows | None, sink: NormSink | None, M: int, N: int, d
 def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tensor | None = None,
            out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
            shuffled: torch.Tensor | None = None, sink: NormSink | None = None,
-           keep_shares: bool = False) -> "torch.Tensor | NormedRows | ShareSum":
+           keep_shares: bool = False, act: str | None = None) -> "torch.Tensor | NormedRows | ShareSum":
     """``a @ weight.T + bias``: a [M, K] (rows may be strided), weight [N, K], bias float32 [N].
     ``shuffled``: the copy of ``weight`` made by :func:`shuffle_weight`, which few-row bfloat16
     products stream instead of ``weight``.  ``a`` may be :class:`NormedRows` and ``sink`` a
     :class:`NormSink` (then the result is the next norm's :class:`NormedRows`); both need the few-row
     kernel (:func:`can_defer_norm` rows, a shuffled copy).  ``keep_shares``: the caller takes a
-    :class:`ShareSum` where the product is computed in shares of K (many rows, a long K)."""
+    :class:`ShareSum` where the product is computed in shares of K (many rows, a long K).  ``act`` "relu2":
+    the result is ``max(y, 0)^2`` in ``out_dtype``, computed in float32: in the few-row bfloat16 kernel's
+    epilogue where that kernel runs the product, by a pass of its own otherwise."""
+    if act is not None:
+        _check(act == "relu2" and not isinstance(a, NormedRows) and sink is None and out is None and not keep_shares,
+               "linear: the activation is 'relu2', on a plain product")
+        M, K = a.shape
+        lda = a.stride(0) if M > 1 else K
+        if (weight.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1 and _skinny_ok(a, shuffled, M, K, lda)
+                and not _few_rows_go_to_rows64(weight.shape[0], K)):
+            _on_gpu(a, weight, bias, shuffled)
+            N = weight.shape[0]
+            _check(weight.shape[1] == K, f"linear: input has K={K}, weight has K={weight.shape[1]}")
+            _check_shuffled(shuffled, N, K)
+            if bias is not None:
+                _check(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == N,
+                       f"linear: bias must be float32 of {N} entries")
+            na = _NormArgs()
+            na.act = 1
+            res = torch.empty(M, N, dtype=out_dtype or a.dtype, device=a.device)
+            _call("tl_gemm_skinny", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(res), _code(res, "linear output"), M, N, K, lda, N,
+                  ctypes.byref(na), _stream())
+            return res
+        return relu_squared(linear(a, weight, bias, out_dtype=torch.float32, shuffled=shuffled), out_dtype or a.dtype)
     owed = a if isinstance(a, NormedRows) else None
     if owed is not None:
         a = owed.rows

@@ -97,9 +97,9 @@ class Linear:
         return self.shuffled if self.shuffled is not None else self.shuffled_float
 
     def __call__(self, x, out_dtype: torch.dtype | None = None, sink=None, with_bias: bool = True,
-                 keep_shares: bool = False):
+                 keep_shares: bool = False, act: str | None = None):
         return kernels.linear(x, self.weight, self.bias if with_bias else None, out_dtype=out_dtype,
-                              shuffled=self.streamed, sink=sink, keep_shares=keep_shares)
+                              shuffled=self.streamed, sink=sink, keep_shares=keep_shares, act=act)
 
 
 def fuse_linears(name: str, parts: list[Linear]) -> Linear:

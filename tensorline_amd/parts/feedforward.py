@@ -55,7 +55,8 @@ class SwiGLU(Part):
 @register_feed_forward("up_down")
 class UpDown(Part):
     """A feed-forward without gate: ``down(act(up(h)))``, no biases.  ``activation``: "relu2", the
-    square of relu, computed in float32.  Tensors under the prefix: up, down."""
+    square of relu, computed in float32 (in the product's epilogue in few-row bfloat16 steps, by a pass
+    of its own otherwise).  Tensors under the prefix: up, down."""
 
     ACTIVATIONS = ("relu2",)
 
@@ -82,5 +83,5 @@ class UpDown(Part):
         return [(self.up.weight, torch.float32), (self.down.weight, torch.float32)]
 
     def forward(self, h, ctx):
-        act = kernels.relu_squared(self.up(h, out_dtype=torch.float32), self.dtype)
+        act = self.up(h, out_dtype=self.dtype, act=self.activation)       # the activation rides on few-row products
         return self.down(act, out_dtype=torch.float32)

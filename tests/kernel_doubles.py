@@ -41,11 +41,13 @@ def shuffle_weight(weight):
     return None
 
 
-def linear(a, weight, bias=None, out_dtype=None, out=None, shuffled=None, sink=None, keep_shares=False):
+def linear(a, weight, bias=None, out_dtype=None, out=None, shuffled=None, sink=None, keep_shares=False, act=None):
     assert sink is None, "the stand-ins make no shuffled copies, so no part defers a norm"
     y = a.to(torch.float32) @ weight.to(torch.float32).T
     if bias is not None:
         y = y + bias
+    if act == "relu2":
+        y = torch.relu(y) ** 2
     return y.to(out_dtype or a.dtype)
 
 
