@@ -1147,6 +1147,9 @@ def batched_linear(a: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) ->
 
 # ---------------------------------------------------------------------------------------------
 # Recurrences over a matrix state per head
+SSD_WALK_MAX_TOKENS = 16    # steps whose sequences bring at most this many tokens walk the state-space form token by token
+
+
 def recurrence_takes_key_dim(dk: int) -> bool:
     return bool(library().tl_linear_recurrence_takes(int(dk)))
 
@@ -1165,7 +1168,9 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ctx, st
     * ``steps`` float32 [T, heads] with ``rate_log`` [heads], ``step_bias`` [heads] and ``skip`` [heads]
       (the last two optional): ``dt = softplus(steps_t + step_bias)``, ``S <- exp(-exp(rate_log) dt) S + dt
       k_t v_t^T``, ``o_t = S^T q_t + skip v_t``; the ``share`` consecutive heads of a group read the same
-      queries and keys (``q``, ``k`` [T, heads / share * dk]).
+      queries and keys (``q``, ``k`` [T, heads / share * dk]).  Steps with prompt portions of more than
+      ``SSD_WALK_MAX_TOKENS`` tokens (``dk`` a multiple of 16 up to 128, ``dv`` up to 128) compute this form in chunks of tokens
+      (``tl_ssd_chunked``): the same sums in another order, so results agree with the walk within rounding.
 
     ``q``, ``k`` [T, heads * dk] and ``v`` [T, heads * dv] are float32 and may be column blocks of a
     wider matrix; ``silu_inputs`` applies SiLU to all three on the way in.  Returns float32 [T, heads * dv]."""
@@ -1196,6 +1201,18 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ctx, st
     st, stride = _state_ptr(state, state_offset)
     out = torch.empty(T, heads * dv, dtype=torch.float32, device=q.device)
     ld = lambda t: t.stride(0) if T > 1 else max(t.shape[1], t.stride(0))
+    facts = getattr(ctx, "facts", None)
+    if (per_token == 2 and facts is not None and not facts.decode_only and facts.max_query_len > SSD_WALK_MAX_TOKENS
+            and library().tl_ssd_chunked_takes(dk, dv)):
+        # prompt portions: chunks of tokens as independent work, the state handed from chunk to chunk by a scan
+        chunks = -(-int(facts.max_query_len) // library().tl_ssd_chunk_tokens())
+        S = ctx.num_seqs
+        ws = torch.empty(S * chunks * heads * (dk * dv + 1), dtype=torch.float32, device=q.device)
+        n_state = S * chunks * heads * dk * dv
+        _call("tl_ssd_chunked", _ptr(q), ld(q), _ptr(k), ld(k), _ptr(v), ld(v), _ptr(steps), ld(steps), _ptr(rate_log),
+              _ptr(step_bias), _ptr(skip), share, st, ctypes.c_longlong(stride), _ptr(ctx.state_slots), _ptr(ctx.q_start),
+              _ptr(out), heads * dv, _ptr(ws[:n_state]), _ptr(ws[n_state:]), S, chunks, heads, dk, dv, _stream())
+        return out
     _call("tl_linear_recurrence", _ptr(q), ld(q), _ptr(k), ld(k), _ptr(v), ld(v), _ptr(wlog), ld(wlog) if per_token else 0,
           _ptr(decay), _ptr(bonus), per_token, _ptr(skip if per_token == 2 else None), share,
           st, ctypes.c_longlong(stride), _ptr(ctx.state_slots),

@@ -475,3 +475,56 @@ def test_a_long_prompt_in_portions_then_decoded_across_the_key_splits(dtype):
     assert len(got) == len(steps)
     for p, row in got.items():
         assert rel_error(row, want[p]) < LIMIT[dtype], f"position {p}: {rel_error(row, want[p]):.3e}"
+
+
+# ---- the state-space recurrence in chunks against the token-by-token walk -----------------------------------------
+@pytest.mark.parametrize("case", [
+    # heads, share, N, P, tokens of each sequence, first column of q and k in their matrix
+    (4, 2, 32, 48, [150, 1, 64], 0),
+    (6, 3, 128, 64, [333, 17], 4),
+    (2, 1, 16, 8, [65, 128, 63, 2], 0),
+    (3, 3, 64, 100, [200], 3),             # value size no multiple of 16; rows that start at no 16-byte border
+    (8, 8, 48, 128, [70, 70], 8),
+])
+def test_state_space_recurrence_in_chunks_equals_the_walk(case, monkeypatch):
+    """Prompt portions compute the state-space form in chunks of 64 tokens on the matrix cores; the walk computes it
+    token by token.  Same operands, states that enter non-zero: outputs and the states left behind agree within
+    float rounding, for chunks that are full, partial and single, several sequences in a step, and operands that
+    are column blocks of wider matrices."""
+    from types import SimpleNamespace
+    from tensorline_amd.engine.batch import StepFacts
+    from tensorline_amd.ops import kernels
+    H, share, N, P, lens, col0 = case
+    G, T = H // share, sum(lens)
+    torch.manual_seed(sum(lens) + N)
+    wide = torch.randn(T, col0 + 2 * G * N + 5, device=DEV)
+    q, k = wide[:, col0:col0 + G * N], wide[:, col0 + G * N:col0 + 2 * G * N]
+    v = torch.randn(T, H * P, device=DEV)
+    steps, rate_log = torch.randn(T, H, device=DEV), torch.randn(H, device=DEV) - 1.0
+    bias, skip = torch.randn(H, device=DEV), torch.randn(H, device=DEV)
+    starts = [0]
+    for n in lens:
+        starts.append(starts[-1] + n)
+    ctx = SimpleNamespace(
+        facts=StepFacts(max_context=max(lens), max_query_len=max(lens), decode_only=False, num_seqs=len(lens), q_lens=list(lens),
+                        starts=[0] * len(lens)),
+        num_seqs=len(lens), state_slots=torch.arange(len(lens), dtype=torch.int32, device=DEV),
+        q_start=torch.tensor(starts, dtype=torch.int32, device=DEV))
+    state0 = torch.randn(len(lens) + 1, H * N * P + 7, device=DEV)
+
+    def run():
+        state = state0.clone()
+        out = kernels.linear_recurrence(q, k, v, ctx, state, H, N, P, steps=steps, rate_log=rate_log, step_bias=bias, skip=skip,
+                                        share=share)
+        return out, state
+    called = []
+    call = kernels._call
+    monkeypatch.setattr(kernels, "_call", lambda name, *a: (called.append(name), call(name, *a))[1])
+    chunked, state_c = run()
+    monkeypatch.setattr(kernels, "SSD_WALK_MAX_TOKENS", 1 << 30)
+    walked, state_w = run()
+    assert called == ["tl_ssd_chunked", "tl_linear_recurrence"]
+    scale = walked.abs().max().item()
+    assert (chunked - walked).abs().max().item() < 2e-5 * scale
+    assert (state_c - state_w).abs().max().item() < 2e-5 * state_w.abs().max().item()
+    assert torch.equal(state_c[:, H * N * P:], state0[:, H * N * P:])         # what lies behind the state is not touched
